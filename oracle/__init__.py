@@ -1,0 +1,170 @@
+"""TEST INFRASTRUCTURE -- numpy front end of the CPU oracle (``libchop_oracle.so``).
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this package.  The product package never does.
+
+Every function takes and returns C-contiguous numpy arrays in the reference op's
+layouts (custom_helper_op/cc/ops/custom_helper_ops.cc:190-307):
+ref ``[B,H,W,C]``, src ``[B,N,srcH,srcW,C]``, base_plane ``[B,H,W,1]``,
+offsets ``[B,D]``, depth_grid ``[B,H,W,D]``, Rs ``[B,N,3,3]``, Ts ``[B,N,3]``,
+cost ``[B,H,W,D,C|G]``, mask int32 ``[B,H,W,D,1]`` (MEAN) or ``[B,H,W,D,C|G]`` (MIN).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libchop_oracle.so")
+_lib = None
+
+MEAN, MIN = 0, 1
+_REDUCE = {"MEAN": 0, "MIN": 1, 0: 0, 1: 1}
+
+
+def build(force=False):
+    """Compile the oracle with the Makefile beside this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "-B"] if force else ["make", "-C", _HERE], check=True,
+                       stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _sfx(dtype):
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return "f32"
+    if dtype == np.float64:
+        return "f64"
+    raise TypeError("oracle computes in float32 or float64 only, got %s" % dtype)
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else ctypes.c_void_p(0)
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def _i64(*v):
+    return [ctypes.c_int64(int(x)) for x in v]
+
+
+def _check(rc, name):
+    if rc != 0:
+        raise ValueError("%s failed with oracle status %d" % (name, rc))
+
+
+def cost_volume_fwd(ref, src, base_plane, offsets, Rs, Ts, reduce="MEAN", half_centor=True,
+                    threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, base_plane, offsets, Rs, Ts = (_c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts))
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = offsets.shape[1]
+    r = _REDUCE[reduce]
+    cost = np.empty((B, H, W, D, C), dt)
+    mask = np.empty((B, H, W, D, 1 if r == 0 else C), np.int32)
+    fn = getattr(lib(), "chop_oracle_cost_volume_fwd_" + sfx)
+    rc = fn(r, int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref), _p(src),
+            _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
+    _check(rc, "cost_volume_fwd")
+    return cost, mask
+
+
+def cost_volume_bwd(ref, src, base_plane, offsets, Rs, Ts, cost_grad, mask, reduce="MEAN",
+                    half_centor=True, threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, base_plane, offsets, Rs, Ts, cost_grad = (
+        _c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts, cost_grad))
+    mask = _c(mask, np.int32)
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = offsets.shape[1]
+    ref_grad = np.empty_like(ref)
+    src_grad = np.empty_like(src)
+    bp_grad = np.empty_like(base_plane)
+    fn = getattr(lib(), "chop_oracle_cost_volume_bwd_" + sfx)
+    rc = fn(_REDUCE[reduce], int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref),
+            _p(src), _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost_grad), _p(mask),
+            _p(ref_grad), _p(src_grad), _p(bp_grad), int(threads))
+    _check(rc, "cost_volume_bwd")
+    return ref_grad, src_grad, bp_grad
+
+
+def cost_volume_v2_fwd(ref, src, depth_grid, Rs, Ts, reduce="MEAN", groups=1, half_centor=True,
+                       threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, depth_grid, Rs, Ts = (_c(x, dt) for x in (ref, src, depth_grid, Rs, Ts))
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = depth_grid.shape[3]
+    r = _REDUCE[reduce]
+    G = int(groups)
+    cost = np.empty((B, H, W, D, max(G, 0)), dt)
+    mask = np.empty((B, H, W, D, 1 if r == 0 else max(G, 0)), np.int32)
+    fn = getattr(lib(), "chop_oracle_cost_volume_v2_fwd_" + sfx)
+    rc = fn(r, int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW, G), _p(ref), _p(src),
+            _p(depth_grid), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
+    _check(rc, "cost_volume_v2_fwd")
+    return cost, mask
+
+
+def cost_volume_v2_bwd(ref, src, depth_grid, Rs, Ts, cost_grad, mask, reduce="MEAN", groups=1,
+                       half_centor=True, threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, depth_grid, Rs, Ts, cost_grad = (
+        _c(x, dt) for x in (ref, src, depth_grid, Rs, Ts, cost_grad))
+    mask = _c(mask, np.int32)
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = depth_grid.shape[3]
+    ref_grad = np.empty_like(ref)
+    src_grad = np.empty_like(src)
+    dg_grad = np.empty_like(depth_grid)
+    fn = getattr(lib(), "chop_oracle_cost_volume_v2_bwd_" + sfx)
+    rc = fn(_REDUCE[reduce], int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW, int(groups)),
+            _p(ref), _p(src), _p(depth_grid), _p(Rs), _p(Ts), _p(cost_grad), _p(mask),
+            _p(ref_grad), _p(src_grad), _p(dg_grad), int(threads))
+    _check(rc, "cost_volume_v2_bwd")
+    return ref_grad, src_grad, dg_grad
+
+
+def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):
+    """Per-(voxel, view) source coordinates ``[B,H,W,D,N]``: (sw, sh, fh, fw, state)."""
+    if depth_grid is not None:
+        dt = depth_grid.dtype
+        depth_grid = _c(depth_grid, dt)
+        B, H, W, D = depth_grid.shape
+        base_plane = offsets = None
+    else:
+        dt = base_plane.dtype
+        base_plane, offsets = _c(base_plane, dt), _c(offsets, dt)
+        B, H, W = base_plane.shape[:3]
+        D = offsets.shape[1]
+    sfx = _sfx(dt)
+    Rs, Ts = _c(Rs, dt), _c(Ts, dt)
+    N = Rs.shape[1]
+    sH, sW = src_hw
+    shape = (B, H, W, D, N)
+    sw, sh = np.empty(shape, dt), np.empty(shape, dt)
+    fh, fw, st = (np.empty(shape, np.int32) for _ in range(3))
+    fn = getattr(lib(), "chop_oracle_sample_coords_" + sfx)
+    rc = fn(int(bool(half_centor)), *_i64(B, H, W, D, N, sH, sW), _p(base_plane), _p(offsets),
+            _p(depth_grid), _p(Rs), _p(Ts), _p(sw), _p(sh), _p(fh), _p(fw), _p(st))
+    _check(rc, "sample_coords")
+    return sw, sh, fh, fw, st
