@@ -1,0 +1,219 @@
+"""Benchmark of the cost-volume hot path on one MI355X.
+
+A step is one forward + one backward of the operator (through the C ABI) on one batch of
+synthetic input that is already resident in HBM.  Prints one JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+class Runner:
+    """Pre-allocated buffers + direct C-ABI calls, so a step enqueues kernels and nothing else."""
+
+    def __init__(self, wl, torch, lib):
+        self.wl, self.torch, self.lib = wl, torch, lib
+        t = wl.tensors
+        td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[wl.storage]
+        self.storage_code = {"f32": 0, "f16": 1, "bf16": 2}[wl.storage]
+        d = "cuda:0"
+        up = lambda k, dt=None: (torch.from_numpy(t[k]).to(d) if dt is None
+                                 else torch.from_numpy(t[k]).to(d).to(dt))
+        self.ref, self.src = up("ref", td), up("src", td)
+        self.Rs, self.Ts = up("Rs"), up("Ts")
+        self.v2 = wl.op == "v2"
+        if self.v2:
+            self.depth_grid = up("depth_grid")
+        else:
+            self.base_plane, self.offsets = up("base_plane"), up("offsets")
+        B, H, W, D, OC = wl.B, wl.H, wl.W, wl.D, wl.out_channels
+        self.cost = torch.empty((B, H, W, D, OC), dtype=td, device=d)
+        self.mask = torch.empty((B, H, W, D, 1), dtype=torch.int32, device=d)
+        gen = torch.Generator(device=d)
+        gen.manual_seed(wl.seed)
+        self.cost_grad = torch.randn((B, H, W, D, OC), dtype=torch.float32, device=d,
+                                     generator=gen).to(td)
+        self.ref_grad = torch.empty_like(self.ref)
+        self.src_grad = torch.empty_like(self.src)
+        self.depth_grad = torch.empty((B, H, W, D) if self.v2 else (B, H, W, 1),
+                                      dtype=torch.float32, device=d)
+        self.dims = (B, H, W, wl.C, D, wl.N, H, W)
+        self.ws = None
+        self.ws_bytes = 0
+        if self.storage_code:
+            self.ws_bytes = lib.chop_cost_volume_bwd16_workspace_bytes(B, H, W, wl.C, wl.N, H, W)
+            self.ws = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=d)
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def forward(self):
+        p = lambda x: x.data_ptr()
+        lib, s = self.lib, self.stream
+        if self.v2:
+            if self.storage_code:
+                rc = lib.chop_cost_volume_v2_fwd_16(s, self.storage_code, 0, 1, *self.dims,
+                                                    self.wl.groups, p(self.ref), p(self.src),
+                                                    p(self.depth_grid), p(self.Rs), p(self.Ts),
+                                                    p(self.cost), p(self.mask))
+            else:
+                rc = lib.chop_cost_volume_v2_fwd_f32(s, 0, 1, *self.dims, self.wl.groups,
+                                                     p(self.ref), p(self.src), p(self.depth_grid),
+                                                     p(self.Rs), p(self.Ts), p(self.cost),
+                                                     p(self.mask))
+        elif self.storage_code:
+            rc = lib.chop_cost_volume_fwd_16(s, self.storage_code, 0, 1, *self.dims, p(self.ref),
+                                             p(self.src), p(self.base_plane), p(self.offsets), None,
+                                             p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
+        else:
+            rc = lib.chop_cost_volume_fwd_f32(s, 0, 1, *self.dims, p(self.ref), p(self.src),
+                                              p(self.base_plane), p(self.offsets), p(self.Rs),
+                                              p(self.Ts), p(self.cost), p(self.mask))
+        if rc:
+            raise RuntimeError(lib.chop_last_error_string().decode())
+
+    def backward(self):
+        p = lambda x: x.data_ptr()
+        lib, s = self.lib, self.stream
+        tail = (p(self.cost_grad), p(self.mask), p(self.ref_grad), p(self.src_grad),
+                p(self.depth_grad))
+        if self.v2:
+            if self.storage_code:
+                rc = lib.chop_cost_volume_v2_bwd_16(s, self.storage_code, 0, 1, *self.dims,
+                                                    self.wl.groups, p(self.ref), p(self.src),
+                                                    p(self.depth_grid), p(self.Rs), p(self.Ts),
+                                                    *tail, p(self.ws), self.ws_bytes)
+            else:
+                rc = lib.chop_cost_volume_v2_bwd_f32(s, 0, 1, *self.dims, self.wl.groups,
+                                                     p(self.ref), p(self.src), p(self.depth_grid),
+                                                     p(self.Rs), p(self.Ts), *tail)
+        elif self.storage_code:
+            rc = lib.chop_cost_volume_bwd_16(s, self.storage_code, 0, 1, *self.dims, p(self.ref),
+                                             p(self.src), p(self.base_plane), p(self.offsets), None,
+                                             p(self.Rs), p(self.Ts), *tail, p(self.ws),
+                                             self.ws_bytes)
+        else:
+            rc = lib.chop_cost_volume_bwd_f32(s, 0, 1, *self.dims, p(self.ref), p(self.src),
+                                              p(self.base_plane), p(self.offsets), p(self.Rs),
+                                              p(self.Ts), *tail)
+        if rc:
+            raise RuntimeError(lib.chop_last_error_string().decode())
+
+
+def cpu_baseline(wl, budget_s=12.0):
+    """The CPU oracle (a port of the reference kernel's per-voxel loop; the reference has
+    no CPU kernel of its own) on the same workload, all host threads the box grants."""
+    import numpy as np
+    import oracle
+    from custom_helper_op_amd.configs import quantise
+    threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")), 16))
+    t = wl.tensors
+    rng = np.random.default_rng(wl.seed)
+    # bounded sample: a horizontal band of the image (all views, all depth hypotheses)
+    rows = wl.H
+    est_voxel_rate = 4.0e6 * threads  # voxel*view*channel/32 per second, conservative
+    work = wl.voxels * wl.N * wl.C / 32.0
+    if work / est_voxel_rate > budget_s:
+        rows = max(8, int(wl.H * budget_s * est_voxel_rate / work))
+    sl = slice(0, rows)
+    ref, src = t["ref"][:, sl], t["src"]
+    cg = quantise(rng.standard_normal((wl.B, rows, wl.W, wl.D, wl.out_channels), dtype=np.float32),
+                  wl.storage)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        if wl.op == "v1":
+            bp = t["base_plane"][:, sl]
+            args = (ref, src, bp, t["offsets"], t["Rs"], t["Ts"])
+            _, mask = oracle.cost_volume_fwd(*args, threads=threads)
+            oracle.cost_volume_bwd(*args, cg, mask, threads=threads)
+        else:
+            dg = t["depth_grid"][:, sl]
+            args = (ref, src, dg, t["Rs"], t["Ts"])
+            _, mask = oracle.cost_volume_v2_fwd(*args, "MEAN", wl.groups, threads=threads)
+            oracle.cost_volume_v2_bwd(*args, cg, mask, "MEAN", wl.groups, threads=threads)
+        times.append(time.perf_counter() - t0)
+        if sum(times) > budget_s:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    vox = wl.B * rows * wl.W * wl.D
+    return {"value": vox / med, "unit": "voxels/s", "cores": threads, "kind": "port",
+            "sample": "%s rows 0..%d of %d (all views, all %d depths), fwd+bwd, median of %d, "
+                      "includes host allocation of outputs" % (wl.name, rows, wl.H, wl.D, len(times))}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", type=int, default=2)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this operator runs on one GPU; --gpus %d is not supported "
+                 "(there is no multi-GPU path to measure)" % a.gpus)
+    import torch
+    from custom_helper_op_amd import _lib
+    from custom_helper_op_amd.configs import make_workload
+    lib = _lib.load()
+    wl = make_workload(a.workload, with_cost_grad=False)
+    r = Runner(wl, torch, lib)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    for _ in range(a.warmup):
+        r.forward()
+        r.backward()
+    torch.cuda.synchronize()
+    marks = []
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        e0, e1, e2 = ev(), ev(), ev()
+        e0.record()
+        r.forward()
+        e1.record()
+        r.backward()
+        e2.record()
+        marks.append((e0, e1, e2))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(m[0].elapsed_time(m[1]) for m in marks) / len(marks)
+    bwd_ms = sum(m[1].elapsed_time(m[2]) for m in marks) / len(marks)
+    ms_per_step = wall * 1e3 / a.steps
+    fwd_b, bwd_b = wl.algorithmic_bytes()
+    dominant = "backward" if bwd_ms >= fwd_ms else "forward"
+    d_ms, d_b = (bwd_ms, bwd_b) if dominant == "backward" else (fwd_ms, fwd_b)
+    achieved = d_b / (d_ms * 1e-3) / 1e9
+    out = {
+        "metric": "cost-volume voxels/s (B*D*H*W) fwd+bwd",
+        "value": wl.voxels / (ms_per_step * 1e-3),
+        "unit": "voxels/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": wl.storage, "data": "synthetic",
+        "config": {"workload": "%s: %s B%d N%d %dx%d C%d D%d%s %s fwd+bwd" % (
+            wl.name, "CostVolume" if wl.op == "v1" else "CostVolumeV2", wl.B, wl.N, wl.H, wl.W,
+            wl.C, wl.D, " G%d" % wl.groups if wl.op == "v2" else "", wl.storage),
+            "voxels": wl.voxels, "reduce_method": "MEAN", "half_centor": True},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": None,
+                     "algorithmic_bytes": {"forward": fwd_b, "backward": bwd_b},
+                     "ms": {"forward": fwd_ms, "backward": bwd_ms},
+                     "fwd_bwd_frac": (fwd_b + bwd_b) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

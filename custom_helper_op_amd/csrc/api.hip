@@ -1,0 +1,395 @@
+// C ABI of libchop_costvol: argument validation, kernel-family selection, error strings.
+// Validation mirrors the checks of the reference's OpKernel::Compute
+// (custom_helper_op/cc/kernels/cost_volume_kernels.cc:91-106, :220-243 and
+// cost_volume_kernels_v2.cc:93-110) as far as they can be expressed on raw pointers and
+// sizes; it runs before any HIP call, so bad arguments are reported on any machine.
+#include <cstdio>
+#include <limits>
+#include <string>
+
+#include "../../include/chop_costvol.h"
+#include "internal.h"
+
+namespace chop {
+namespace {
+
+thread_local std::string g_last_error = "";
+thread_local int g_kernel_family = 0;
+
+int fail(int code, const std::string &msg) {
+  g_last_error = msg;
+  return code;
+}
+
+struct Dims {
+  int64_t B, H, W, C, D, N, srcH, srcW;
+};
+
+bool mul_overflows(std::initializer_list<int64_t> f, int64_t *out) {
+  __int128 p = 1;
+  for (int64_t v : f) {
+    p *= v;
+    if (p > (__int128)std::numeric_limits<int64_t>::max() / 16) return true;
+  }
+  *out = (int64_t)p;
+  return false;
+}
+
+// Returns 0 or an error code.  Sets *empty when no kernel has to run.
+int check_dims(const Dims &d, int reduce, int groups, bool correlation) {
+  if (d.B < 0 || d.H < 0 || d.W < 0 || d.C < 0 || d.D < 0 || d.N < 0 || d.srcH < 0 || d.srcW < 0)
+    return fail(CHOP_ERR_BAD_DIMS, "negative dimension");
+  const int64_t lim = std::numeric_limits<int32_t>::max();
+  if (d.H > lim || d.W > lim || d.C > lim || d.D > lim || d.N > lim || d.srcH > lim ||
+      d.srcW > lim || d.B > lim)
+    return fail(CHOP_ERR_BAD_DIMS, "a single dimension exceeds 2^31-1");
+  int64_t tmp;
+  if (mul_overflows({d.B, d.H, d.W, d.D, d.C > 0 ? d.C : 1}, &tmp) ||
+      mul_overflows({d.B, d.N, d.srcH, d.srcW, d.C > 0 ? d.C : 1}, &tmp))
+    return fail(CHOP_ERR_BAD_DIMS, "tensor element count overflows");
+  if (reduce != CHOP_REDUCE_MEAN && reduce != CHOP_REDUCE_MIN)
+    return fail(CHOP_ERR_BAD_ENUM, "reduce must be CHOP_REDUCE_MEAN (0) or CHOP_REDUCE_MIN (1)");
+  if (correlation && (groups <= 0 || d.C % groups != 0))
+    return fail(CHOP_ERR_BAD_GROUPS, "groups must be positive and divide the channel count");
+  return 0;
+}
+
+#define REQUIRE_PTR(p, count)                                                          \
+  do {                                                                                 \
+    if ((p) == nullptr && (count) > 0)                                                 \
+      return fail(CHOP_ERR_NULL_POINTER, std::string("null pointer: ") + #p);          \
+  } while (0)
+
+int launch_status(hipError_t err, const char *what) {
+  if (err == hipSuccess) return CHOP_OK;
+  return fail(CHOP_ERR_LAUNCH, std::string(what) + ": " + hipGetErrorString(err));
+}
+
+template <typename S>
+int forward(void *stream, int reduce, int half_centor, const Dims &d, int groups, int corr,
+            const S *ref, const S *src, const typename Storage<S>::Real *base_plane,
+            const typename Storage<S>::Real *offsets, const typename Storage<S>::Real *depth_grid,
+            const typename Storage<S>::Real *Rs, const typename Storage<S>::Real *Ts, S *cost,
+            int32_t *mask, bool needs_depth_grid) {
+  using R = typename Storage<S>::Real;
+  if (int rc = check_dims(d, reduce, groups, corr == GROUP_CORRELATION)) return rc;
+  const int64_t pixels = d.B * d.H * d.W, voxels = pixels * d.D;
+  const int64_t oc = corr == GROUP_CORRELATION ? groups : d.C;
+  if (voxels == 0 || oc == 0) return CHOP_OK;  // nothing to write
+  REQUIRE_PTR(ref, pixels * d.C);
+  REQUIRE_PTR(src, d.B * d.N * d.srcH * d.srcW * d.C);
+  if (needs_depth_grid || depth_grid != nullptr) {
+    REQUIRE_PTR(depth_grid, voxels);
+  } else {
+    REQUIRE_PTR(base_plane, pixels);
+    REQUIRE_PTR(offsets, d.B * d.D);
+  }
+  REQUIRE_PTR(Rs, d.B * d.N);
+  REQUIRE_PTR(Ts, d.B * d.N);
+  REQUIRE_PTR(cost, voxels);
+  REQUIRE_PTR(mask, voxels);
+  Args<S> a{};
+  a.B = d.B, a.H = d.H, a.W = d.W, a.C = d.C, a.D = d.D, a.N = d.N, a.srcH = d.srcH, a.srcW = d.srcW;
+  a.groups = corr == GROUP_CORRELATION ? groups : 1;
+  a.reduce = reduce, a.corr = corr, a.half = half_centor ? R(0.5) : R(0);
+  a.ref = ref, a.src = src, a.base_plane = base_plane, a.offsets = offsets;
+  a.depth_grid = depth_grid, a.Rs = Rs, a.Ts = Ts, a.cost = cost, a.mask = mask;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (g_kernel_family == 0 && tiled_forward_supported(a))
+    return launch_status(launch_tiled_forward(a, s), "tiled forward launch");
+  return launch_status(launch_general_forward(a, s), "general forward launch");
+}
+
+template <typename S>
+int backward(void *stream, int reduce, int half_centor, const Dims &d, int groups, int corr,
+             const S *ref, const S *src, const typename Storage<S>::Real *base_plane,
+             const typename Storage<S>::Real *offsets,
+             const typename Storage<S>::Real *depth_grid, const typename Storage<S>::Real *Rs,
+             const typename Storage<S>::Real *Ts, const S *cost_grad, const int32_t *mask,
+             S *ref_grad, S *src_grad, typename Storage<S>::Real *depth_grad,
+             bool needs_depth_grid, void *workspace, size_t workspace_bytes) {
+  using R = typename Storage<S>::Real;
+  if (int rc = check_dims(d, reduce, groups, corr == GROUP_CORRELATION)) return rc;
+  const int64_t pixels = d.B * d.H * d.W, voxels = pixels * d.D;
+  const int64_t n_ref = pixels * d.C, n_src = d.B * d.N * d.srcH * d.srcW * d.C;
+  const bool per_voxel_depth = needs_depth_grid || depth_grid != nullptr;
+  const int64_t n_depth = per_voxel_depth ? voxels : pixels;
+  if (n_ref == 0 && n_src == 0 && n_depth == 0) return CHOP_OK;
+  REQUIRE_PTR(ref_grad, n_ref);
+  REQUIRE_PTR(src_grad, n_src);
+  REQUIRE_PTR(depth_grad, n_depth);
+  const bool work = voxels > 0 && d.C > 0;
+  if (work) {
+    REQUIRE_PTR(ref, n_ref);
+    REQUIRE_PTR(src, n_src);
+    if (per_voxel_depth) {
+      REQUIRE_PTR(depth_grid, voxels);
+    } else {
+      REQUIRE_PTR(base_plane, pixels);
+      REQUIRE_PTR(offsets, d.B * d.D);
+    }
+    REQUIRE_PTR(Rs, d.B * d.N);
+    REQUIRE_PTR(Ts, d.B * d.N);
+    REQUIRE_PTR(cost_grad, voxels);
+    REQUIRE_PTR(mask, voxels);
+  }
+  Args<S> a{};
+  a.B = d.B, a.H = d.H, a.W = d.W, a.C = d.C, a.D = d.D, a.N = d.N, a.srcH = d.srcH, a.srcW = d.srcW;
+  a.groups = corr == GROUP_CORRELATION ? groups : 1;
+  a.reduce = reduce, a.corr = corr, a.half = half_centor ? R(0.5) : R(0);
+  a.ref = ref, a.src = src, a.base_plane = base_plane, a.offsets = offsets;
+  a.depth_grid = depth_grid, a.Rs = Rs, a.Ts = Ts;
+  a.cost_grad = cost_grad, a.mask_in = mask;
+  a.ref_grad = ref_grad, a.src_grad = src_grad, a.depth_grad = depth_grad;
+  if (sizeof(S) == 2) {
+    const size_t need = chop_cost_volume_bwd16_workspace_bytes(d.B, d.H, d.W, d.C, d.N, d.srcH, d.srcW);
+    if (need > 0) {
+      if (workspace == nullptr) return fail(CHOP_ERR_WORKSPACE, "workspace is null");
+      if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+        return fail(CHOP_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+      if (workspace_bytes < need) {
+        char buf[128];
+        snprintf(buf, sizeof buf, "workspace too small: %zu bytes given, %zu needed",
+                 workspace_bytes, need);
+        return fail(CHOP_ERR_WORKSPACE, buf);
+      }
+    }
+    a.src_grad_acc = static_cast<float *>(workspace);
+    a.ref_grad_acc = a.src_grad_acc + ((n_src + 63) / 64) * 64;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (g_kernel_family == 0 && work && tiled_backward_supported(a))
+    return launch_status(launch_tiled_backward(a, s), "tiled backward launch");
+  return launch_status(launch_general_backward(a, s), "general backward launch");
+}
+
+}  // namespace
+}  // namespace chop
+
+using namespace chop;
+
+extern "C" {
+
+int chop_abi_version(void) { return 1; }
+
+const char *chop_last_error_string(void) { return g_last_error.c_str(); }
+
+int chop_set_kernel_family(int family) {
+  const int prev = g_kernel_family;
+  g_kernel_family = family == 1 ? 1 : 0;
+  return prev;
+}
+
+#define DIMS \
+  Dims { B, H, W, C, D, N, srcH, srcW }
+
+int chop_cost_volume_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const float *ref, const float *src,
+                             const float *base_plane, const float *offsets, const float *Rs,
+                             const float *Ts, float *cost, int32_t *mask) {
+  return forward<float>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE, ref, src,
+                        base_plane, offsets, nullptr, Rs, Ts, cost, mask, false);
+}
+
+int chop_cost_volume_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const double *ref, const double *src,
+                             const double *base_plane, const double *offsets, const double *Rs,
+                             const double *Ts, double *cost, int32_t *mask) {
+  return forward<double>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE, ref, src,
+                         base_plane, offsets, nullptr, Rs, Ts, cost, mask, false);
+}
+
+int chop_cost_volume_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const float *ref, const float *src,
+                             const float *base_plane, const float *offsets, const float *Rs,
+                             const float *Ts, const float *cost_grad, const int32_t *mask,
+                             float *ref_grad, float *src_grad, float *base_plane_grad) {
+  return backward<float>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE, ref, src,
+                         base_plane, offsets, nullptr, Rs, Ts, cost_grad, mask, ref_grad, src_grad,
+                         base_plane_grad, false, nullptr, 0);
+}
+
+int chop_cost_volume_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const double *ref, const double *src,
+                             const double *base_plane, const double *offsets, const double *Rs,
+                             const double *Ts, const double *cost_grad, const int32_t *mask,
+                             double *ref_grad, double *src_grad, double *base_plane_grad) {
+  return backward<double>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE, ref, src,
+                          base_plane, offsets, nullptr, Rs, Ts, cost_grad, mask, ref_grad,
+                          src_grad, base_plane_grad, false, nullptr, 0);
+}
+
+int chop_cost_volume_v2_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const float *ref, const float *src,
+                                const float *depth_grid, const float *Rs, const float *Ts,
+                                float *cost, int32_t *mask) {
+  return forward<float>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION, ref, src,
+                        nullptr, nullptr, depth_grid, Rs, Ts, cost, mask, true);
+}
+
+int chop_cost_volume_v2_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const double *ref, const double *src,
+                                const double *depth_grid, const double *Rs, const double *Ts,
+                                double *cost, int32_t *mask) {
+  return forward<double>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION, ref, src,
+                         nullptr, nullptr, depth_grid, Rs, Ts, cost, mask, true);
+}
+
+int chop_cost_volume_v2_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const float *ref, const float *src,
+                                const float *depth_grid, const float *Rs, const float *Ts,
+                                const float *cost_grad, const int32_t *mask, float *ref_grad,
+                                float *src_grad, float *depth_grid_grad) {
+  return backward<float>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION, ref, src,
+                         nullptr, nullptr, depth_grid, Rs, Ts, cost_grad, mask, ref_grad,
+                         src_grad, depth_grid_grad, true, nullptr, 0);
+}
+
+int chop_cost_volume_v2_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const double *ref, const double *src,
+                                const double *depth_grid, const double *Rs, const double *Ts,
+                                const double *cost_grad, const int32_t *mask, double *ref_grad,
+                                double *src_grad, double *depth_grid_grad) {
+  return backward<double>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION, ref, src,
+                          nullptr, nullptr, depth_grid, Rs, Ts, cost_grad, mask, ref_grad,
+                          src_grad, depth_grid_grad, true, nullptr, 0);
+}
+
+size_t chop_cost_volume_bwd16_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C,
+                                              int64_t N, int64_t srcH, int64_t srcW) {
+  if (B < 0 || H < 0 || W < 0 || C < 0 || N < 0 || srcH < 0 || srcW < 0) return 0;
+  const int64_t n_src = B * N * srcH * srcW * C, n_ref = B * H * W * C;
+  return (size_t)(((n_src + 63) / 64) * 64 + ((n_ref + 63) / 64) * 64) * sizeof(float);
+}
+
+#define STORAGE_DISPATCH(expr_half, expr_bf16)                                              \
+  switch (storage) {                                                                        \
+    case CHOP_STORAGE_F16:                                                                  \
+      return expr_half;                                                                     \
+    case CHOP_STORAGE_BF16:                                                                 \
+      return expr_bf16;                                                                     \
+    default:                                                                                \
+      return fail(CHOP_ERR_BAD_ENUM, "storage must be CHOP_STORAGE_F16 or CHOP_STORAGE_BF16"); \
+  }
+
+int chop_cost_volume_fwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                            int64_t H, int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                            int64_t srcW, const void *ref, const void *src,
+                            const float *base_plane, const float *offsets,
+                            const float *depth_grid, const float *Rs, const float *Ts,
+                            void *cost, int32_t *mask) {
+  STORAGE_DISPATCH(
+      forward<__half>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE,
+                      (const __half *)ref, (const __half *)src, base_plane, offsets, depth_grid,
+                      Rs, Ts, (__half *)cost, mask, false),
+      forward<bf16_t>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE,
+                      (const bf16_t *)ref, (const bf16_t *)src, base_plane, offsets, depth_grid,
+                      Rs, Ts, (bf16_t *)cost, mask, false))
+}
+
+int chop_cost_volume_bwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                            int64_t H, int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                            int64_t srcW, const void *ref, const void *src,
+                            const float *base_plane, const float *offsets,
+                            const float *depth_grid, const float *Rs, const float *Ts,
+                            const void *cost_grad, const int32_t *mask, void *ref_grad,
+                            void *src_grad, float *depth_grad, void *workspace,
+                            size_t workspace_bytes) {
+  STORAGE_DISPATCH(
+      backward<__half>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE,
+                       (const __half *)ref, (const __half *)src, base_plane, offsets, depth_grid,
+                       Rs, Ts, (const __half *)cost_grad, mask, (__half *)ref_grad,
+                       (__half *)src_grad, depth_grad, false, workspace, workspace_bytes),
+      backward<bf16_t>(stream, reduce, half_centor, DIMS, 1, SQUARED_DIFFERENCE,
+                       (const bf16_t *)ref, (const bf16_t *)src, base_plane, offsets, depth_grid,
+                       Rs, Ts, (const bf16_t *)cost_grad, mask, (bf16_t *)ref_grad,
+                       (bf16_t *)src_grad, depth_grad, false, workspace, workspace_bytes))
+}
+
+int chop_cost_volume_v2_fwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                               int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                               int64_t srcH, int64_t srcW, int groups, const void *ref,
+                               const void *src, const float *depth_grid, const float *Rs,
+                               const float *Ts, void *cost, int32_t *mask) {
+  STORAGE_DISPATCH(
+      forward<__half>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
+                      (const __half *)ref, (const __half *)src, nullptr, nullptr, depth_grid, Rs,
+                      Ts, (__half *)cost, mask, true),
+      forward<bf16_t>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
+                      (const bf16_t *)ref, (const bf16_t *)src, nullptr, nullptr, depth_grid, Rs,
+                      Ts, (bf16_t *)cost, mask, true))
+}
+
+int chop_cost_volume_v2_bwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                               int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                               int64_t srcH, int64_t srcW, int groups, const void *ref,
+                               const void *src, const float *depth_grid, const float *Rs,
+                               const float *Ts, const void *cost_grad, const int32_t *mask,
+                               void *ref_grad, void *src_grad, float *depth_grid_grad,
+                               void *workspace, size_t workspace_bytes) {
+  STORAGE_DISPATCH(
+      backward<__half>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
+                       (const __half *)ref, (const __half *)src, nullptr, nullptr, depth_grid, Rs,
+                       Ts, (const __half *)cost_grad, mask, (__half *)ref_grad,
+                       (__half *)src_grad, depth_grid_grad, true, workspace, workspace_bytes),
+      backward<bf16_t>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
+                       (const bf16_t *)ref, (const bf16_t *)src, nullptr, nullptr, depth_grid, Rs,
+                       Ts, (const bf16_t *)cost_grad, mask, (bf16_t *)ref_grad,
+                       (bf16_t *)src_grad, depth_grid_grad, true, workspace, workspace_bytes))
+}
+
+int chop_cost_volume_sample_coords_f32(void *stream, int half_centor, int64_t B, int64_t H,
+                                       int64_t W, int64_t D, int64_t N, int64_t srcH,
+                                       int64_t srcW, const float *base_plane,
+                                       const float *offsets, const float *depth_grid,
+                                       const float *Rs, const float *Ts, float *sw, float *sh,
+                                       int32_t *fh, int32_t *fw, int32_t *state) {
+  const Dims d{B, H, W, 1, D, N, srcH, srcW};
+  if (int rc = check_dims(d, 0, 1, false)) return rc;
+  const int64_t total = B * H * W * D * N;
+  if (total == 0) return CHOP_OK;
+  if (depth_grid == nullptr) {
+    REQUIRE_PTR(base_plane, total);
+    REQUIRE_PTR(offsets, total);
+  }
+  REQUIRE_PTR(Rs, total); REQUIRE_PTR(Ts, total); REQUIRE_PTR(sw, total); REQUIRE_PTR(sh, total);
+  REQUIRE_PTR(fh, total); REQUIRE_PTR(fw, total); REQUIRE_PTR(state, total);
+  return launch_status(
+      launch_sample_coords<float>(half_centor ? 0.5f : 0.f, B, H, W, D, N, srcH, srcW, base_plane,
+                                  offsets, depth_grid, Rs, Ts, sw, sh, fh, fw, state,
+                                  static_cast<hipStream_t>(stream)),
+      "sample_coords launch");
+}
+
+int chop_cost_volume_sample_coords_f64(void *stream, int half_centor, int64_t B, int64_t H,
+                                       int64_t W, int64_t D, int64_t N, int64_t srcH,
+                                       int64_t srcW, const double *base_plane,
+                                       const double *offsets, const double *depth_grid,
+                                       const double *Rs, const double *Ts, double *sw,
+                                       double *sh, int32_t *fh, int32_t *fw, int32_t *state) {
+  const Dims d{B, H, W, 1, D, N, srcH, srcW};
+  if (int rc = check_dims(d, 0, 1, false)) return rc;
+  const int64_t total = B * H * W * D * N;
+  if (total == 0) return CHOP_OK;
+  if (depth_grid == nullptr) {
+    REQUIRE_PTR(base_plane, total);
+    REQUIRE_PTR(offsets, total);
+  }
+  REQUIRE_PTR(Rs, total); REQUIRE_PTR(Ts, total); REQUIRE_PTR(sw, total); REQUIRE_PTR(sh, total);
+  REQUIRE_PTR(fh, total); REQUIRE_PTR(fw, total); REQUIRE_PTR(state, total);
+  return launch_status(
+      launch_sample_coords<double>(half_centor ? 0.5 : 0.0, B, H, W, D, N, srcH, srcW, base_plane,
+                                   offsets, depth_grid, Rs, Ts, sw, sh, fh, fw, state,
+                                   static_cast<hipStream_t>(stream)),
+      "sample_coords launch");
+}
+
+}  // extern "C"

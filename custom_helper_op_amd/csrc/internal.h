@@ -1,0 +1,75 @@
+// Host-side plumbing shared by the C ABI (api.hip) and the kernel families
+// (general.hip, tiled.hip): the argument block and the launcher prototypes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "warp.h"
+
+namespace chop {
+
+enum Corr { SQUARED_DIFFERENCE = 0, GROUP_CORRELATION = 1 };
+
+// One call's arguments after validation.  S = storage type of the feature tensors,
+// R = Storage<S>::Real = type of depth inputs, camera matrices, depth gradients.
+template <typename S>
+struct Args {
+  using R = typename Storage<S>::Real;
+  int64_t B, H, W, C, D, N, srcH, srcW;
+  int groups;        // 1 for the squared-difference op
+  int reduce;        // CHOP_REDUCE_MEAN / CHOP_REDUCE_MIN
+  int corr;          // Corr
+  R half;            // 0.5 or 0
+  const S *ref, *src;
+  const R *base_plane, *offsets;  // depth = base_plane[pixel] + offsets[b,d] ...
+  const R *depth_grid;            // ... unless depth_grid != nullptr: depth_grid[voxel]
+  const R *Rs, *Ts;
+  // forward
+  S *cost;
+  int32_t *mask;
+  // backward
+  const S *cost_grad;
+  const int32_t *mask_in;
+  S *ref_grad, *src_grad;
+  R *depth_grad;  // [B,H,W] (base_plane) or [B,H,W,D] (depth_grid)
+  // fp32 accumulation images for 16-bit storage (nullptr otherwise)
+  float *ref_grad_acc, *src_grad_acc;
+
+  __host__ __device__ int64_t pixels() const { return B * H * W; }
+  __host__ __device__ int64_t voxels() const { return B * H * W * D; }
+  __host__ __device__ int out_channels() const { return corr == GROUP_CORRELATION ? groups : (int)C; }
+};
+
+// General kernels: any shape, any channel count, both reduces, all storage types.
+template <typename S>
+hipError_t launch_general_forward(const Args<S> &a, hipStream_t stream);
+template <typename S>
+hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream);
+
+// Tiled kernels: wavefront-per-pixel-tile, depth innermost.  `supported` says whether the
+// shape qualifies; the launchers must only be called when it does.
+template <typename S>
+bool tiled_forward_supported(const Args<S> &a);
+template <typename S>
+hipError_t launch_tiled_forward(const Args<S> &a, hipStream_t stream);
+template <typename S>
+bool tiled_backward_supported(const Args<S> &a);
+template <typename S>
+hipError_t launch_tiled_backward(const Args<S> &a, hipStream_t stream);
+
+// Utility launches.
+hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+template <typename S>
+hipError_t launch_narrow(const float *from, S *to, int64_t count, hipStream_t stream);
+
+template <typename R>
+hipError_t launch_sample_coords(R half, int64_t B, int64_t H, int64_t W, int64_t D, int64_t N,
+                                int64_t srcH, int64_t srcW, const R *base_plane,
+                                const R *offsets, const R *depth_grid, const R *Rs, const R *Ts,
+                                R *sw, R *sh, int32_t *fh, int32_t *fw, int32_t *state,
+                                hipStream_t stream);
+
+int grid_for(int64_t work_items, int block);
+
+}  // namespace chop

@@ -1,0 +1,320 @@
+"""Host-side mirror of the reference's Python operator interface for the cost volume.
+
+Same names, argument order, defaults and outputs as
+custom_helper_op/python/ops/custom_helper_ops.py:32-96 (``cost_volume``,
+``cost_volume_v2`` and the gradients registered for them), with torch tensors standing in
+for TensorFlow tensors: torch supplies device memory and the current HIP stream, the
+arithmetic is done by ``libchop_costvol.so`` through its C ABI.  The shape checks are the
+ones ``CostVolumeOp::Compute`` performs (custom_helper_op/cc/kernels/
+cost_volume_kernels.cc:91-106, :220-243; cost_volume_kernels_v2.cc:93-110), raised as
+``InvalidArgumentError``.
+
+float32/float64 follow the registered ops; float16/bfloat16 feature tensors use the
+library's 16-bit storage extension (depth inputs and camera matrices must then be
+float32).
+"""
+import torch
+
+from . import _lib
+
+_REDUCE = {"MEAN": 0, "MIN": 1}
+_STORAGE16 = {torch.float16: 1, torch.bfloat16: 2}
+
+
+class InvalidArgumentError(ValueError):
+    """What ``OP_REQUIRES(..., errors::InvalidArgument(...))`` becomes on this side."""
+
+
+def _reduce_code(reduce_method):
+    if reduce_method not in _REDUCE:
+        # the reference aborts the process here (LOG(FATAL), cost_volume_kernels.cc:71)
+        raise InvalidArgumentError(
+            "Invalid reduce method %r. Supported types: MEAN, MIN" % (reduce_method,))
+    return _REDUCE[reduce_method]
+
+
+def _require(cond, msg):
+    if not cond:
+        raise InvalidArgumentError(msg)
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _prep(t, dtype, device, name):
+    t = torch.as_tensor(t)
+    _require(t.dtype == dtype, "%s must have dtype %s, got %s" % (name, dtype, t.dtype))
+    _require(t.device == device, "%s must live on %s" % (name, device))
+    return t.contiguous()
+
+
+def _real_dtype(dtype):
+    _require(dtype in (torch.float32, torch.float64, torch.float16, torch.bfloat16),
+             "dtype must be float32 or float64 (float16/bfloat16 storage as an extension)")
+    return torch.float32 if dtype in _STORAGE16 else dtype
+
+
+def _check_common(ref_image, src_images, Rs, Ts):
+    _require(ref_image.dim() == 4, "ref image must have rank 4")
+    B, H, W, C = ref_image.shape
+    _require(src_images.dim() == 5 and src_images.shape[0] == B and src_images.shape[2] == H
+             and src_images.shape[3] == W and src_images.shape[4] == C,
+             "src_images must have rank 5, and must compate to ref_image")
+    N = src_images.shape[1]
+    _require(Rs.dim() == 4 and tuple(Rs.shape) == (B, N, 3, 3),
+             "Rs must have rank 2, and must compate to ref_image")
+    _require(Ts.dim() == 3 and tuple(Ts.shape) == (B, N, 3),
+             "Ts must have rank 2, and must compate to ref_image")
+    return B, H, W, C, N
+
+
+def _check_v1(ref_image, src_images, base_plane, offsets, Rs, Ts):
+    B, H, W, C, N = _check_common(ref_image, src_images, Rs, Ts)
+    _require(base_plane.dim() == 4 and tuple(base_plane.shape) == (B, H, W, 1),
+             "base_plane must have rank 4, and must compate to ref_image")
+    _require(offsets.dim() == 2 and offsets.shape[0] == B,
+             "offsets must have rank 2, and must compate to ref_image")
+    return B, H, W, C, N, offsets.shape[1]
+
+
+def _check_v2(ref_image, src_images, depth_grid, Rs, Ts, groups):
+    B, H, W, C, N = _check_common(ref_image, src_images, Rs, Ts)
+    _require(depth_grid.dim() == 4 and tuple(depth_grid.shape[:3]) == (B, H, W),
+             "depth_grid must have rank 4, and must compate to ref_image")
+    _require(isinstance(groups, int) and groups > 0 and C % groups == 0,
+             "image_channels must be divisible by groups")
+    return B, H, W, C, N, depth_grid.shape[3]
+
+
+def cost_volume_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
+                    half_centor=True):
+    """Forward op without autograd: returns ``(cost [B,H,W,D,C], cost_mask int32)``."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    rdt = _real_dtype(dt)
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, rdt, dev, "base_plane")
+    offsets = _prep(offsets, rdt, dev, "offsets")
+    Rs, Ts = _prep(Rs, rdt, dev, "Rs"), _prep(Ts, rdt, dev, "Ts")
+    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, Rs, Ts)
+    cost = torch.empty((B, H, W, D, C), dtype=dt, device=dev)
+    mask = torch.empty((B, H, W, D, 1 if red == 0 else C), dtype=torch.int32, device=dev)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    if dt in _STORAGE16:
+        rc = lib.chop_cost_volume_fwd_16(_stream(cost), _STORAGE16[dt], red, int(half_centor), *dims,
+                                         _ptr(ref_image), _ptr(src_images), _ptr(base_plane),
+                                         _ptr(offsets), None, _ptr(Rs), _ptr(Ts), _ptr(cost),
+                                         _ptr(mask))
+    else:
+        fn = lib.chop_cost_volume_fwd_f32 if dt == torch.float32 else lib.chop_cost_volume_fwd_f64
+        rc = fn(_stream(cost), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
+                _ptr(base_plane), _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(cost), _ptr(mask))
+    _lib.check(rc)
+    return cost, mask
+
+
+def cost_volume_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_grad, cost_mask,
+                     reduce_method="MEAN", half_centor=True):
+    """The ``CostVolumeGrad`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    rdt = _real_dtype(dt)
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, rdt, dev, "base_plane")
+    offsets = _prep(offsets, rdt, dev, "offsets")
+    rs, ts = _prep(rs, rdt, dev, "Rs"), _prep(ts, rdt, dev, "Ts")
+    cost_grad = _prep(cost_grad, dt, dev, "cost_grad")
+    cost_mask = _prep(cost_mask, torch.int32, dev, "cost_mask")
+    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, rs, ts)
+    _require(tuple(cost_grad.shape) == (B, H, W, D, C),
+             "cost_grad must have rank 5, and must compate to ref_image")
+    _require(tuple(cost_mask.shape) == (B, H, W, D, 1 if red == 0 else C),
+             "cost_mask must have rank 5, and must compate to ref_image")
+    ref_grad = torch.empty_like(ref_image)
+    src_grad = torch.empty_like(src_images)
+    bp_grad = torch.empty_like(base_plane)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    if dt in _STORAGE16:
+        need = lib.chop_cost_volume_bwd16_workspace_bytes(B, H, W, C, N, *dims[6:])
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        rc = lib.chop_cost_volume_bwd_16(_stream(ref_grad), _STORAGE16[dt], red, int(half_centor),
+                                         *dims, _ptr(ref_image), _ptr(src_images),
+                                         _ptr(base_plane), _ptr(offsets), None, _ptr(rs), _ptr(ts),
+                                         _ptr(cost_grad), _ptr(cost_mask), _ptr(ref_grad),
+                                         _ptr(src_grad), _ptr(bp_grad), _ptr(ws), need)
+    else:
+        fn = lib.chop_cost_volume_bwd_f32 if dt == torch.float32 else lib.chop_cost_volume_bwd_f64
+        rc = fn(_stream(ref_grad), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
+                _ptr(base_plane), _ptr(offsets), _ptr(rs), _ptr(ts), _ptr(cost_grad),
+                _ptr(cost_mask), _ptr(ref_grad), _ptr(src_grad), _ptr(bp_grad))
+    _lib.check(rc)
+    return ref_grad, src_grad, bp_grad
+
+
+def cost_volume_v2_raw(ref_image, src_images, depth_grid, Rs, Ts, reduce_method="MEAN", groups=None,
+                       half_centor=True):
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    rdt = _real_dtype(dt)
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    depth_grid = _prep(depth_grid, rdt, dev, "depth_grid")
+    Rs, Ts = _prep(Rs, rdt, dev, "Rs"), _prep(Ts, rdt, dev, "Ts")
+    B, H, W, C, N, D = _check_v2(ref_image, src_images, depth_grid, Rs, Ts, groups)
+    cost = torch.empty((B, H, W, D, groups), dtype=dt, device=dev)
+    mask = torch.empty((B, H, W, D, 1 if red == 0 else groups), dtype=torch.int32, device=dev)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    if dt in _STORAGE16:
+        rc = lib.chop_cost_volume_v2_fwd_16(_stream(cost), _STORAGE16[dt], red, int(half_centor),
+                                            *dims, groups, _ptr(ref_image), _ptr(src_images),
+                                            _ptr(depth_grid), _ptr(Rs), _ptr(Ts), _ptr(cost),
+                                            _ptr(mask))
+    else:
+        fn = (lib.chop_cost_volume_v2_fwd_f32 if dt == torch.float32
+              else lib.chop_cost_volume_v2_fwd_f64)
+        rc = fn(_stream(cost), red, int(half_centor), *dims, groups, _ptr(ref_image),
+                _ptr(src_images), _ptr(depth_grid), _ptr(Rs), _ptr(Ts), _ptr(cost), _ptr(mask))
+    _lib.check(rc)
+    return cost, mask
+
+
+def cost_volume_grad_v2(ref_image, src_images, depth_grid, rs, ts, cost_grad, cost_mask,
+                        reduce_method="MEAN", groups=None, half_centor=True):
+    """The ``CostVolumeGradV2`` op: ``(ref_image_grad, src_images_grad, depth_grid_grad)``."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    rdt = _real_dtype(dt)
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    depth_grid = _prep(depth_grid, rdt, dev, "depth_grid")
+    rs, ts = _prep(rs, rdt, dev, "Rs"), _prep(ts, rdt, dev, "Ts")
+    cost_grad = _prep(cost_grad, dt, dev, "cost_grad")
+    cost_mask = _prep(cost_mask, torch.int32, dev, "cost_mask")
+    B, H, W, C, N, D = _check_v2(ref_image, src_images, depth_grid, rs, ts, groups)
+    _require(tuple(cost_grad.shape) == (B, H, W, D, groups),
+             "cost_grad must have rank 5, and must compate to ref_image")
+    _require(tuple(cost_mask.shape) == (B, H, W, D, 1 if red == 0 else groups),
+             "cost_mask must have rank 5, and must compate to ref_image")
+    ref_grad = torch.empty_like(ref_image)
+    src_grad = torch.empty_like(src_images)
+    dg_grad = torch.empty_like(depth_grid)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    if dt in _STORAGE16:
+        need = lib.chop_cost_volume_bwd16_workspace_bytes(B, H, W, C, N, *dims[6:])
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        rc = lib.chop_cost_volume_v2_bwd_16(_stream(ref_grad), _STORAGE16[dt], red,
+                                            int(half_centor), *dims, groups, _ptr(ref_image),
+                                            _ptr(src_images), _ptr(depth_grid), _ptr(rs), _ptr(ts),
+                                            _ptr(cost_grad), _ptr(cost_mask), _ptr(ref_grad),
+                                            _ptr(src_grad), _ptr(dg_grad), _ptr(ws), need)
+    else:
+        fn = (lib.chop_cost_volume_v2_bwd_f32 if dt == torch.float32
+              else lib.chop_cost_volume_v2_bwd_f64)
+        rc = fn(_stream(ref_grad), red, int(half_centor), *dims, groups, _ptr(ref_image),
+                _ptr(src_images), _ptr(depth_grid), _ptr(rs), _ptr(ts), _ptr(cost_grad),
+                _ptr(cost_mask), _ptr(ref_grad), _ptr(src_grad), _ptr(dg_grad))
+    _lib.check(rc)
+    return ref_grad, src_grad, dg_grad
+
+
+class _CostVolume(torch.autograd.Function):
+    """Forward = CostVolume, backward = the gradient registered for it
+    (custom_helper_ops.py:41-61): the Grad op is fed the forward's cost_mask, the incoming
+    gradient of cost_mask is ignored, offsets/Rs/Ts receive no gradient."""
+
+    @staticmethod
+    def forward(ctx, ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method, half_centor):
+        cost, mask = cost_volume_raw(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                     reduce_method, half_centor)
+        ctx.save_for_backward(ref_image, src_images, base_plane, offsets, Rs, Ts, mask)
+        ctx.attrs = (reduce_method, half_centor)
+        ctx.mark_non_differentiable(mask)
+        return cost, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        ref_image, src_images, base_plane, offsets, Rs, Ts, mask = ctx.saved_tensors
+        rg, sg, bg = cost_volume_grad(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                      grad_out.contiguous(), mask, *ctx.attrs)
+        return rg, sg, bg, None, None, None, None, None
+
+
+class _CostVolumeV2(torch.autograd.Function):
+    """CostVolumeV2 with its registered gradient (custom_helper_ops.py:74-94)."""
+
+    @staticmethod
+    def forward(ctx, ref_image, src_images, depth_grid, Rs, Ts, reduce_method, groups, half_centor):
+        cost, mask = cost_volume_v2_raw(ref_image, src_images, depth_grid, Rs, Ts, reduce_method,
+                                        groups, half_centor)
+        ctx.save_for_backward(ref_image, src_images, depth_grid, Rs, Ts, mask)
+        ctx.attrs = (reduce_method, groups, half_centor)
+        ctx.mark_non_differentiable(mask)
+        return cost, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        ref_image, src_images, depth_grid, Rs, Ts, mask = ctx.saved_tensors
+        rg, sg, dg = cost_volume_grad_v2(ref_image, src_images, depth_grid, Rs, Ts,
+                                         grad_out.contiguous(), mask, *ctx.attrs)
+        return rg, sg, dg, None, None, None, None, None
+
+
+def cost_volume(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
+                half_centor=True, name=None):
+    """``custom_helper_op.cost_volume``: returns ``(cost, cost_mask)``; differentiable with
+    respect to ref_image, src_images and base_plane."""
+    del name
+    offsets = torch.as_tensor(offsets, device=ref_image.device)
+    Rs = torch.as_tensor(Rs, device=ref_image.device)
+    Ts = torch.as_tensor(Ts, device=ref_image.device)
+    return _CostVolume.apply(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method,
+                             half_centor)
+
+
+def cost_volume_v2(ref_image, src_images, depth_grid, Rs, Ts, reduce_method="MEAN", groups=None,
+                   half_centor=True, name=None):
+    """``custom_helper_op.cost_volume_v2``: returns ``(cost [B,H,W,D,groups], cost_mask)``."""
+    del name
+    depth_grid = torch.as_tensor(depth_grid, device=ref_image.device)
+    Rs = torch.as_tensor(Rs, device=ref_image.device)
+    Ts = torch.as_tensor(Ts, device=ref_image.device)
+    return _CostVolumeV2.apply(ref_image, src_images, depth_grid, Rs, Ts, reduce_method, groups,
+                               half_centor)
+
+
+def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):
+    """Diagnostic: per-(voxel, view) sample coordinates ``[B,H,W,D,N]`` as the kernels
+    compute them: ``(sw, sh, fh, fw, state)``."""
+    lib = _lib.load()
+    if depth_grid is not None:
+        dt, dev = depth_grid.dtype, depth_grid.device
+        depth_grid = depth_grid.contiguous()
+        B, H, W, D = depth_grid.shape
+    else:
+        dt, dev = base_plane.dtype, base_plane.device
+        base_plane, offsets = base_plane.contiguous(), offsets.contiguous()
+        B, H, W = base_plane.shape[:3]
+        D = offsets.shape[1]
+    Rs, Ts = _prep(Rs, dt, dev, "Rs"), _prep(Ts, dt, dev, "Ts")
+    N = Rs.shape[1]
+    shape = (B, H, W, D, N)
+    sw, sh = (torch.empty(shape, dtype=dt, device=dev) for _ in range(2))
+    fh, fw, st = (torch.empty(shape, dtype=torch.int32, device=dev) for _ in range(3))
+    fn = (lib.chop_cost_volume_sample_coords_f32 if dt == torch.float32
+          else lib.chop_cost_volume_sample_coords_f64)
+    rc = fn(_stream(sw), int(half_centor), B, H, W, D, N, src_hw[0], src_hw[1], _ptr(base_plane),
+            _ptr(offsets), _ptr(depth_grid), _ptr(Rs), _ptr(Ts), _ptr(sw), _ptr(sh), _ptr(fh),
+            _ptr(fw), _ptr(st))
+    _lib.check(rc)
+    return sw, sh, fh, fw, st

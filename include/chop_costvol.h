@@ -1,0 +1,191 @@
+/*
+ * libchop_costvol -- plane-sweep cost-volume operator for AMD MI355X (gfx950), C ABI.
+ *
+ * Drop-in replacement for the device functors of zhuimeng999/custom_helper_op's
+ * CostVolume / CostVolumeGrad / CostVolumeV2 / CostVolumeGradV2 ops.  Every entry
+ * point takes plain device pointers and sizes, enqueues work on the given HIP stream
+ * and returns immediately; it never synchronises and never allocates or frees device
+ * memory.  The caller owns every buffer.  Gradient outputs may arrive uninitialised:
+ * the library clears what it accumulates into.
+ *
+ * Tensor layouts (dense, row-major, innermost last), as registered by the reference
+ * (custom_helper_op/cc/ops/custom_helper_ops.cc:190-307):
+ *   ref        [B,H,W,C]            src        [B,N,srcH,srcW,C]
+ *   base_plane [B,H,W,1]            offsets    [B,D]            (V1 depth = base + offset)
+ *   depth_grid [B,H,W,D]                                          (V2 depth)
+ *   Rs         [B,N,3,3]  = K_src R K_ref^-1        Ts [B,N,3] = K_src t
+ *   cost       [B,H,W,D,C] (V1)  /  [B,H,W,D,groups] (V2)
+ *   mask int32 [B,H,W,D,1] for CHOP_REDUCE_MEAN (valid-view count)
+ *              [B,H,W,D,C|groups] for CHOP_REDUCE_MIN (winning view or -1)
+ *   gradients shaped like ref, src, base_plane (V1) / depth_grid (V2).
+ *
+ * Return value: 0 on success, a chop_status otherwise; chop_last_error_string()
+ * describes the last failure on the calling thread.  Zero-sized work is a successful
+ * no-op (the reference aborts on it, cost_volume_kernels_gpu.cu.cc:238).
+ * All entry points are re-entrant and may be called from several host threads.
+ */
+#ifndef CHOP_COSTVOL_H_
+#define CHOP_COSTVOL_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum chop_status {
+  CHOP_OK = 0,
+  CHOP_ERR_NULL_POINTER = 1,   /* a required buffer is NULL */
+  CHOP_ERR_BAD_DIMS = 2,       /* negative or overflowing dimension */
+  CHOP_ERR_BAD_ENUM = 3,       /* reduce is neither CHOP_REDUCE_MEAN nor CHOP_REDUCE_MIN */
+  CHOP_ERR_BAD_GROUPS = 4,     /* groups <= 0 or C % groups != 0 */
+  CHOP_ERR_LAUNCH = 5,         /* HIP reported an error when the work was enqueued */
+  CHOP_ERR_WORKSPACE = 6,      /* workspace NULL, misaligned or too small */
+  CHOP_ERR_NO_DEVICE = 7       /* no usable HIP device */
+} chop_status;
+
+/* reduce_method attr of the ops: "MEAN" / "MIN"
+ * (reference enum COST_REDUCE_METHOD, custom_helper_op/cc/kernels/cost_volume.h:35). */
+enum { CHOP_REDUCE_MEAN = 0, CHOP_REDUCE_MIN = 1 };
+
+/* Element types of the 16-bit storage extension. */
+enum { CHOP_STORAGE_F16 = 1, CHOP_STORAGE_BF16 = 2 };
+
+int chop_abi_version(void);
+const char *chop_last_error_string(void);
+
+/* ---- CostVolume forward ------------------------------------------------------------
+ * Replaces functor::CostVolumeFunctor<GPUDevice,T,half_centor>::operator()
+ * (declared custom_helper_op/cc/kernels/cost_volume.h:37-80, defined
+ * cost_volume_kernels_gpu.cu.cc:289-335, called from CostVolumeOp::Compute,
+ * cost_volume_kernels.cc:128-136).  `stream` is a hipStream_t. */
+int chop_cost_volume_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const float *ref, const float *src,
+                             const float *base_plane, const float *offsets, const float *Rs,
+                             const float *Ts, float *cost, int32_t *mask);
+int chop_cost_volume_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const double *ref, const double *src,
+                             const double *base_plane, const double *offsets, const double *Rs,
+                             const double *Ts, double *cost, int32_t *mask);
+
+/* ---- CostVolume backward -----------------------------------------------------------
+ * Replaces functor::CostVolumeGradFunctor<GPUDevice,T,half_centor>::operator()
+ * (cost_volume.h:82-133, cost_volume_kernels_gpu.cu.cc:590-655, called from
+ * CostVolumeGradOp::Compute, cost_volume_kernels.cc:263-271), including the three
+ * SetZeroBig launches (:637-642). */
+int chop_cost_volume_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const float *ref, const float *src,
+                             const float *base_plane, const float *offsets, const float *Rs,
+                             const float *Ts, const float *cost_grad, const int32_t *mask,
+                             float *ref_grad, float *src_grad, float *base_plane_grad);
+int chop_cost_volume_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                             int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                             int64_t srcW, const double *ref, const double *src,
+                             const double *base_plane, const double *offsets, const double *Rs,
+                             const double *Ts, const double *cost_grad, const int32_t *mask,
+                             double *ref_grad, double *src_grad, double *base_plane_grad);
+
+/* ---- CostVolumeV2 forward / backward ------------------------------------------------
+ * Replace functor::CostVolumeV2Functor / CostVolumeGradV2Functor
+ * (custom_helper_op/cc/kernels/cost_volume_v2.h:37-133,
+ * cost_volume_kernels_gpu_v2.cu.cc:296-342 and :614-680, called from
+ * cost_volume_kernels_v2.cc:130-138 and :265-273).  The third gradient is the
+ * depth_grid gradient (registered under the name base_plane_grad,
+ * custom_helper_ops.cc:301); voxels skipped by the mask receive 0. */
+int chop_cost_volume_v2_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const float *ref, const float *src,
+                                const float *depth_grid, const float *Rs, const float *Ts,
+                                float *cost, int32_t *mask);
+int chop_cost_volume_v2_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const double *ref, const double *src,
+                                const double *depth_grid, const double *Rs, const double *Ts,
+                                double *cost, int32_t *mask);
+int chop_cost_volume_v2_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const float *ref, const float *src,
+                                const float *depth_grid, const float *Rs, const float *Ts,
+                                const float *cost_grad, const int32_t *mask, float *ref_grad,
+                                float *src_grad, float *depth_grid_grad);
+int chop_cost_volume_v2_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const double *ref, const double *src,
+                                const double *depth_grid, const double *Rs, const double *Ts,
+                                const double *cost_grad, const int32_t *mask, double *ref_grad,
+                                double *src_grad, double *depth_grid_grad);
+
+/* ---- 16-bit storage extension --------------------------------------------------------
+ * No counterpart in the reference, whose ops register float32 and float64 only
+ * (custom_helper_ops.cc:197,234).  ref, src, cost, cost_grad, ref_grad and src_grad
+ * hold IEEE half (CHOP_STORAGE_F16) or bfloat16 (CHOP_STORAGE_BF16) elements; depth
+ * inputs, camera matrices and depth gradients stay float; coordinates and all
+ * arithmetic are fp32, identical to the f32 entry points run on the widened inputs.
+ * `depth_grid` non-NULL selects per-pixel hypotheses for the V1 squared-difference
+ * reduce (base_plane/offsets are then ignored and the third gradient has the shape of
+ * depth_grid).
+ * The backward accumulates source/reference gradients in fp32 inside `workspace`
+ * (device memory, 256-byte aligned, at least chop_cost_volume_bwd16_workspace_bytes). */
+size_t chop_cost_volume_bwd16_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C,
+                                              int64_t N, int64_t srcH, int64_t srcW);
+int chop_cost_volume_fwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                            int64_t H, int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                            int64_t srcW, const void *ref, const void *src,
+                            const float *base_plane, const float *offsets,
+                            const float *depth_grid, const float *Rs, const float *Ts,
+                            void *cost, int32_t *mask);
+int chop_cost_volume_bwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                            int64_t H, int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                            int64_t srcW, const void *ref, const void *src,
+                            const float *base_plane, const float *offsets,
+                            const float *depth_grid, const float *Rs, const float *Ts,
+                            const void *cost_grad, const int32_t *mask, void *ref_grad,
+                            void *src_grad, float *depth_grad, void *workspace,
+                            size_t workspace_bytes);
+int chop_cost_volume_v2_fwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                               int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                               int64_t srcH, int64_t srcW, int groups, const void *ref,
+                               const void *src, const float *depth_grid, const float *Rs,
+                               const float *Ts, void *cost, int32_t *mask);
+int chop_cost_volume_v2_bwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
+                               int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                               int64_t srcH, int64_t srcW, int groups, const void *ref,
+                               const void *src, const float *depth_grid, const float *Rs,
+                               const float *Ts, const void *cost_grad, const int32_t *mask,
+                               void *ref_grad, void *src_grad, float *depth_grid_grad,
+                               void *workspace, size_t workspace_bytes);
+
+/* ---- diagnostics ------------------------------------------------------------------------
+ * No counterpart in the reference.  Writes, for every (voxel, view), the source-view
+ * sample coordinate exactly as the kernels above compute it, so that coordinates,
+ * truncated indices and acceptance can be compared bit for bit with another
+ * implementation.  Outputs are [B,H,W,D,N]: sw/sh the coordinates (0 when the point is
+ * behind the camera), fh/fw the truncated indices (-1 unless accepted), state 0 behind
+ * the camera, 1 outside the open rectangle (0,srcW-1)x(0,srcH-1), 2 accepted.
+ * depth_grid non-NULL selects the V2 depth source. */
+int chop_cost_volume_sample_coords_f32(void *stream, int half_centor, int64_t B, int64_t H,
+                                       int64_t W, int64_t D, int64_t N, int64_t srcH,
+                                       int64_t srcW, const float *base_plane,
+                                       const float *offsets, const float *depth_grid,
+                                       const float *Rs, const float *Ts, float *sw, float *sh,
+                                       int32_t *fh, int32_t *fw, int32_t *state);
+int chop_cost_volume_sample_coords_f64(void *stream, int half_centor, int64_t B, int64_t H,
+                                       int64_t W, int64_t D, int64_t N, int64_t srcH,
+                                       int64_t srcW, const double *base_plane,
+                                       const double *offsets, const double *depth_grid,
+                                       const double *Rs, const double *Ts, double *sw,
+                                       double *sh, int32_t *fh, int32_t *fw, int32_t *state);
+
+/* Selects the kernel family for subsequent calls from this thread: 0 = automatic
+ * (tiled kernels where the shape allows, otherwise the general kernels), 1 = general
+ * kernels only.  Returns the previous value.  Used by the tests to cover both. */
+int chop_set_kernel_family(int family);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CHOP_COSTVOL_H_ */

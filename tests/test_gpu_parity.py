@@ -1,0 +1,313 @@
+"""GPU parity: the HIP library (through its C ABI) against the CPU oracle on identical
+seeded inputs.  Bars: sample coordinates, truncated indices, acceptance and masks
+bit-exact; fp32 forward values within 1e-5 relative; fp32 backward within 1e-4 relative;
+16-bit storage within 1e-2."""
+import numpy as np
+import pytest
+import torch
+
+import custom_helper_op_amd as chop
+from custom_helper_op_amd import _lib
+from custom_helper_op_amd.configs import make_workload, quantise, reference_test_case
+from gpu_util import (TORCH_DTYPE, assert_backward_close, assert_forward_close, dev, host, rms)
+
+pytestmark = pytest.mark.gpu
+
+FAMILIES = [pytest.param(1, id="general"), pytest.param(0, id="auto")]
+
+
+@pytest.fixture(autouse=True)
+def _announce(request):
+    print("\n[case] %s" % request.node.nodeid, flush=True)
+    yield
+    _lib.load().chop_set_kernel_family(0)
+
+
+def _v1_inputs(t, dtype=None):
+    keys = ("ref", "src", "base_plane", "offsets", "Rs", "Ts")
+    return [dev(t[k].astype(dtype) if dtype else t[k]) for k in keys]
+
+
+# ---- coordinates ---------------------------------------------------------------------------
+@pytest.mark.parametrize("index,hw", [(1, None), (5, (48, 64))])
+@pytest.mark.parametrize("half", [True, False])
+def test_sample_coordinates_bit_exact(oracle, index, hw, half):
+    wl = make_workload(index, hw=hw, with_cost_grad=False, batch=1)
+    t = wl.tensors
+    want = oracle.sample_coords(t["base_plane"], t["offsets"], t["Rs"], t["Ts"], (wl.H, wl.W), half)
+    got = chop.sample_coords(dev(t["base_plane"]), dev(t["offsets"]), dev(t["Rs"]), dev(t["Ts"]),
+                             (wl.H, wl.W), half)
+    names = ("sw", "sh", "fh", "fw", "state")
+    for n, g, w in zip(names, got, want):
+        g = host(g)
+        assert g.dtype == w.dtype
+        assert np.array_equal(g.view(np.int32), w.view(np.int32)), n  # bit patterns
+    assert 0.02 < (want[4] == 2).mean() < 1.0
+
+
+def test_sample_coordinates_bit_exact_f64_and_depth_grid(oracle):
+    t = reference_test_case(3, 2, 3, 12, 16, 3, 6, np.float64, seed=8)
+    want = oracle.sample_coords(t["base_plane"], t["offsets"], t["Rs"], t["Ts"], (12, 16))
+    got = chop.sample_coords(dev(t["base_plane"]), dev(t["offsets"]), dev(t["Rs"]), dev(t["Ts"]),
+                             (12, 16))
+    for g, w in zip(got, want):
+        assert np.array_equal(host(g), w)
+    wl = make_workload(4, hw=(32, 40), with_cost_grad=False, batch=1)
+    dg = wl.tensors["depth_grid"]
+    want = oracle.sample_coords(None, None, wl.tensors["Rs"], wl.tensors["Ts"], (32, 40),
+                                depth_grid=dg)
+    got = chop.sample_coords(None, None, dev(wl.tensors["Rs"]), dev(wl.tensors["Ts"]), (32, 40),
+                             depth_grid=dev(dg))
+    for g, w in zip(got, want):
+        assert np.array_equal(host(g).view(np.int32), w.view(np.int32))
+
+
+# ---- V1 forward ----------------------------------------------------------------------------
+REF_SHAPES = [(1, 1, 12, 16, 3, 5), (1, 2, 12, 16, 3, 9), (2, 2, 12, 18, 5, 10), (2, 3, 12, 16, 3, 6)]
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("shape", REF_SHAPES)
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_v1_forward_reference_shapes(oracle, family, shape, reduce, dtype):
+    """The reference unit tests' shapes and four camera cases (cost_volume_op_test.py:174-263)."""
+    _lib.load().chop_set_kernel_family(family)
+    B, N, H, W, C, D = shape
+    for case in range(4):
+        t = reference_test_case(case, B, N, H, W, C, D, dtype, seed=case)
+        want_cost, want_mask = oracle.cost_volume_fwd(**t, reduce=reduce)
+        cost, mask = chop.cost_volume_raw(*_v1_inputs(t), reduce)
+        assert np.array_equal(host(mask), want_mask)
+        if family == 1:
+            assert np.array_equal(host(cost), want_cost)  # literal operation order: same bits
+        else:
+            assert_forward_close(host(cost), want_cost)
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("half", [True, False])
+def test_v1_forward_tiny_config_full(oracle, family, half):
+    """Benchmark configuration 1 at full size, forward only."""
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(1)
+    t = wl.tensors
+    want_cost, want_mask = oracle.cost_volume_fwd(t["ref"], t["src"], t["base_plane"], t["offsets"],
+                                                  t["Rs"], t["Ts"], "MEAN", half, threads=8)
+    cost, mask = chop.cost_volume_raw(*_v1_inputs(t), "MEAN", half)
+    assert cost.shape == (1, 64, 80, 32, 8) and mask.shape == (1, 64, 80, 32, 1)
+    assert np.array_equal(host(mask), want_mask)
+    assert_forward_close(host(cost), want_cost)
+    assert (want_mask == wl.N).mean() > 0.5
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("index,hw,depth", [(2, (32, 40), None), (5, (36, 48), 32)])
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+def test_v1_forward_benchmark_shapes(oracle, family, index, hw, depth, reduce):
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(index, hw=hw, depth=depth, with_cost_grad=False, batch=min(2, _SPEC_B[index]))
+    t = wl.tensors
+    want_cost, want_mask = oracle.cost_volume_fwd(t["ref"], t["src"], t["base_plane"], t["offsets"],
+                                                  t["Rs"], t["Ts"], reduce, threads=8)
+    cost, mask = chop.cost_volume_raw(*_v1_inputs(t), reduce)
+    assert np.array_equal(host(mask), want_mask)
+    assert_forward_close(host(cost), want_cost)
+
+
+_SPEC_B = {1: 1, 2: 1, 3: 1, 4: 2, 5: 4}
+
+
+# ---- V1 backward ---------------------------------------------------------------------------
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("shape", REF_SHAPES)
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_v1_backward_reference_shapes(oracle, family, shape, reduce, dtype):
+    _lib.load().chop_set_kernel_family(family)
+    B, N, H, W, C, D = shape
+    rng = np.random.default_rng(17)
+    for case in (1, 3):
+        t = reference_test_case(case, B, N, H, W, C, D, dtype, seed=case)
+        _, mask = oracle.cost_volume_fwd(**t, reduce=reduce)
+        cg = rng.standard_normal((B, H, W, D, C)).astype(dtype)
+        want = oracle.cost_volume_bwd(**t, cost_grad=cg, mask=mask, reduce=reduce)
+        got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), dev(mask), reduce)
+        tol = 1e-4 if dtype == np.float32 else 1e-10
+        for g, w in zip(got, want):
+            assert g.shape == w.shape
+            assert_backward_close(host(g), w, tol)
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("index,hw,depth", [(2, (32, 40), None), (5, (36, 48), 32)])
+def test_v1_backward_benchmark_shapes(oracle, family, index, hw, depth):
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(index, hw=hw, depth=depth, batch=min(2, _SPEC_B[index]))
+    t = wl.tensors
+    args = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+    _, mask = oracle.cost_volume_fwd(*args, threads=8)
+    want = oracle.cost_volume_bwd(*args, t["cost_grad"], mask, threads=1)
+    # the same sums accumulated in float64 show how far fp32 summation order alone moves them
+    a64 = tuple(x.astype(np.float64) for x in args)
+    exact = oracle.cost_volume_bwd(*a64, t["cost_grad"].astype(np.float64), mask, threads=8)
+    got = chop.cost_volume_grad(*_v1_inputs(t), dev(t["cost_grad"]), dev(mask))
+    for g, w, e in zip(got, want, exact):
+        assert_backward_close(host(g), w)
+        assert_backward_close(host(g), e.astype(np.float32))
+    # conservation: ref_grad and src_grad cancel in sum (each g enters as -g and as four
+    # taps whose weights sum to one)
+    rg, sg = host(got[0]).astype(np.float64), host(got[1]).astype(np.float64)
+    assert abs(rg.sum() + sg.sum()) < 1e-4 * np.abs(rg).sum()
+
+
+# ---- V2 ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_v2_forward_backward_reference_shapes(oracle, family, reduce, dtype):
+    """cost_volume_v2_op_test.py:174-263: C=9, groups=3, depth_grid = base + offsets."""
+    _lib.load().chop_set_kernel_family(family)
+    rng = np.random.default_rng(23)
+    for (B, N, H, W, D) in [(1, 1, 12, 16, 5), (1, 2, 12, 16, 9), (2, 2, 12, 18, 10), (2, 3, 12, 16, 6)]:
+        for case in (0, 1, 3):
+            t = reference_test_case(case, B, N, H, W, 9, D, dtype, seed=case + 40)
+            dg = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(dtype)
+            want_cost, want_mask = oracle.cost_volume_v2_fwd(t["ref"], t["src"], dg, t["Rs"],
+                                                             t["Ts"], reduce, 3)
+            ins = [dev(t["ref"]), dev(t["src"]), dev(dg), dev(t["Rs"]), dev(t["Ts"])]
+            cost, mask = chop.cost_volume_v2_raw(*ins, reduce, 3)
+            assert np.array_equal(host(mask), want_mask)
+            if family == 1:
+                assert np.array_equal(host(cost), want_cost)
+            else:
+                assert_forward_close(host(cost), want_cost, atol=1e-5)
+            cg = rng.standard_normal(want_cost.shape).astype(dtype)
+            want = oracle.cost_volume_v2_bwd(t["ref"], t["src"], dg, t["Rs"], t["Ts"], cg,
+                                             want_mask, reduce, 3)
+            got = chop.cost_volume_grad_v2(*ins, dev(cg), dev(want_mask), reduce, 3)
+            tol = 1e-4 if dtype == np.float32 else 1e-10
+            for g, w in zip(got, want):
+                assert_backward_close(host(g), w, tol)
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+def test_v2_groupwise_config_f32(oracle, family):
+    """Benchmark configuration 4's shape family (C=8, groups=4, D=8 per-pixel hypotheses)
+    in float32 at reduced resolution."""
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(4, hw=(64, 80), batch=2)
+    t = wl.tensors
+    want_cost, want_mask = oracle.cost_volume_v2_fwd(t["ref"], t["src"], t["depth_grid"], t["Rs"],
+                                                     t["Ts"], "MEAN", 4, threads=8)
+    ins = [dev(t[k]) for k in ("ref", "src", "depth_grid", "Rs", "Ts")]
+    cost, mask = chop.cost_volume_v2_raw(*ins, "MEAN", 4)
+    assert np.array_equal(host(mask), want_mask)
+    assert_forward_close(host(cost), want_cost, atol=1e-5)
+    want = oracle.cost_volume_v2_bwd(t["ref"], t["src"], t["depth_grid"], t["Rs"], t["Ts"],
+                                     t["cost_grad"], want_mask, "MEAN", 4)
+    got = chop.cost_volume_grad_v2(*ins, dev(t["cost_grad"]), dev(want_mask), "MEAN", 4)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+
+
+# ---- 16-bit storage ------------------------------------------------------------------------
+def _assert_16bit_close(got, want, storage):
+    """1e-2 relative, floor 1e-2 * rms: the output itself is rounded to 8 (bf16) or 11
+    (fp16) significant bits."""
+    np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2 * max(rms(want), 1e-30))
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("storage", ["f16", "bf16"])
+def test_v1_16bit_storage(oracle, family, storage):
+    """Benchmark configuration 3's shape family (C=16, N=4, D=32, smooth base plane):
+    fp32 oracle on the quantised inputs, 1e-2."""
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(3, hw=(48, 64))
+    t = wl.tensors
+    ref, src, cg = (quantise(t[k], storage) for k in ("ref", "src", "cost_grad"))
+    want_cost, want_mask = oracle.cost_volume_fwd(ref, src, t["base_plane"], t["offsets"], t["Rs"],
+                                                  t["Ts"], threads=8)
+    td = TORCH_DTYPE[storage]
+    ins = [dev(ref, td), dev(src, td), dev(t["base_plane"]), dev(t["offsets"]), dev(t["Rs"]),
+           dev(t["Ts"])]
+    cost, mask = chop.cost_volume_raw(*ins)
+    assert cost.dtype == td
+    assert np.array_equal(host(mask), want_mask)
+    _assert_16bit_close(host(cost), want_cost, storage)
+    want = oracle.cost_volume_bwd(ref, src, t["base_plane"], t["offsets"], t["Rs"], t["Ts"], cg,
+                                  want_mask)
+    got = chop.cost_volume_grad(*ins, dev(cg, td), dev(want_mask))
+    assert got[0].dtype == td and got[1].dtype == td and got[2].dtype == torch.float32
+    for g, w in zip(got, want):
+        _assert_16bit_close(host(g), w, storage)
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("storage", ["bf16", "f16"])
+def test_v2_16bit_storage(oracle, family, storage):
+    """Benchmark configuration 4 (bf16 group-wise correlation) at reduced resolution."""
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(4, hw=(64, 80), batch=2)
+    t = wl.tensors
+    ref, src, cg = (quantise(t[k], storage) for k in ("ref", "src", "cost_grad"))
+    want_cost, want_mask = oracle.cost_volume_v2_fwd(ref, src, t["depth_grid"], t["Rs"], t["Ts"],
+                                                     "MEAN", 4, threads=8)
+    td = TORCH_DTYPE[storage]
+    ins = [dev(ref, td), dev(src, td), dev(t["depth_grid"]), dev(t["Rs"]), dev(t["Ts"])]
+    cost, mask = chop.cost_volume_v2_raw(*ins, "MEAN", 4)
+    assert np.array_equal(host(mask), want_mask)
+    _assert_16bit_close(host(cost), want_cost, storage)
+    want = oracle.cost_volume_v2_bwd(ref, src, t["depth_grid"], t["Rs"], t["Ts"], cg, want_mask,
+                                     "MEAN", 4)
+    got = chop.cost_volume_grad_v2(*ins, dev(cg, td), dev(want_mask), "MEAN", 4)
+    for g, w in zip(got, want):
+        _assert_16bit_close(host(g), w, storage)
+
+
+# ---- the registered gradient, end to end ------------------------------------------------------
+def test_autograd_matches_grad_op(oracle):
+    """forward -> keep cost_mask -> Grad op with the upstream gradient, the call pattern
+    of the gradient registered in custom_helper_ops.py:41-61."""
+    wl = make_workload(2, hw=(16, 20), depth=24)
+    t = wl.tensors
+    ins = _v1_inputs(t)
+    for x in ins[:3]:
+        x.requires_grad_(True)
+    cost, mask = chop.cost_volume(*ins)
+    assert not mask.requires_grad
+    cg = dev(t["cost_grad"])
+    (cost * cg).sum().backward()
+    _, m = oracle.cost_volume_fwd(t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+    want = oracle.cost_volume_bwd(t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"],
+                                  t["Ts"], t["cost_grad"], m)
+    for x, w in zip(ins[:3], want):
+        assert_backward_close(host(x.grad), w)
+    assert ins[3].grad is None and ins[4].grad is None and ins[5].grad is None
+
+
+def test_empty_and_degenerate_inputs():
+    z = lambda *s: torch.zeros(*s, device="cuda")
+    cost, mask = chop.cost_volume_raw(z(1, 0, 4, 3), z(1, 2, 0, 4, 3), z(1, 0, 4, 1), z(1, 5),
+                                      z(1, 2, 3, 3), z(1, 2, 3))
+    assert cost.shape == (1, 0, 4, 5, 3) and mask.shape == (1, 0, 4, 5, 1)
+    # no source views: every count is zero and the cost row stays zero
+    ref = torch.randn(1, 4, 5, 3, device="cuda")
+    cost, mask = chop.cost_volume_raw(ref, z(1, 0, 4, 5, 3), torch.ones(1, 4, 5, 1, device="cuda"),
+                                      torch.ones(1, 2, device="cuda"), z(1, 0, 3, 3), z(1, 0, 3))
+    assert int(mask.abs().sum()) == 0 and float(cost.abs().sum()) == 0
+    rg, sg, bg = chop.cost_volume_grad(ref, z(1, 0, 4, 5, 3), torch.ones(1, 4, 5, 1, device="cuda"),
+                                       torch.ones(1, 2, device="cuda"), z(1, 0, 3, 3), z(1, 0, 3),
+                                       torch.ones_like(cost), mask)
+    assert float(rg.abs().sum()) == 0 and float(bg.abs().sum()) == 0 and sg.numel() == 0
+    # every sample behind the camera
+    src = torch.randn(1, 2, 4, 5, 3, device="cuda")
+    Rs = torch.eye(3, device="cuda").expand(1, 2, 3, 3).contiguous()
+    Ts = torch.tensor([0.0, 0.0, -100.0], device="cuda").expand(1, 2, 3).contiguous()
+    cost, mask = chop.cost_volume_raw(ref, src, torch.ones(1, 4, 5, 1, device="cuda"),
+                                      torch.ones(1, 2, device="cuda"), Rs, Ts)
+    assert int(mask.abs().sum()) == 0 and float(cost.abs().sum()) == 0
+    cmin, mmin = chop.cost_volume_raw(ref, src, torch.ones(1, 4, 5, 1, device="cuda"),
+                                      torch.ones(1, 2, device="cuda"), Rs, Ts, "MIN")
+    assert bool((mmin == -1).all()) and bool((cmin == torch.finfo(torch.float32).max).all())
