@@ -148,13 +148,9 @@ def test_v1_backward_benchmark_shapes(oracle, family, index, hw, depth):
     args = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
     _, mask = oracle.cost_volume_fwd(*args, threads=8)
     want = oracle.cost_volume_bwd(*args, t["cost_grad"], mask, threads=1)
-    # the same sums accumulated in float64 show how far fp32 summation order alone moves them
-    a64 = tuple(x.astype(np.float64) for x in args)
-    exact = oracle.cost_volume_bwd(*a64, t["cost_grad"].astype(np.float64), mask, threads=8)
     got = chop.cost_volume_grad(*_v1_inputs(t), dev(t["cost_grad"]), dev(mask))
-    for g, w, e in zip(got, want, exact):
+    for g, w in zip(got, want):
         assert_backward_close(host(g), w)
-        assert_backward_close(host(g), e.astype(np.float32))
     # conservation: ref_grad and src_grad cancel in sum (each g enters as -g and as four
     # taps whose weights sum to one)
     rg, sg = host(got[0]).astype(np.float64), host(got[1]).astype(np.float64)
