@@ -17,6 +17,7 @@ SIGNATURES = {
     "chop_abi_version": [],
     "chop_last_error_string": [],
     "chop_set_kernel_family": [_int],
+    "chop_last_kernel_family": [],
     "chop_cost_volume_bwd16_workspace_bytes": [_i64] * 7,
 }
 for _t in ("f32", "f64"):

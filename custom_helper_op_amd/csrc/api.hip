@@ -15,6 +15,7 @@ namespace {
 
 thread_local std::string g_last_error = "";
 thread_local int g_kernel_family = 0;
+thread_local int g_last_family = 0;
 
 int fail(int code, const std::string &msg) {
   g_last_error = msg;
@@ -95,8 +96,11 @@ int forward(void *stream, int reduce, int half_centor, const Dims &d, int groups
   a.ref = ref, a.src = src, a.base_plane = base_plane, a.offsets = offsets;
   a.depth_grid = depth_grid, a.Rs = Rs, a.Ts = Ts, a.cost = cost, a.mask = mask;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (g_kernel_family == 0 && tiled_forward_supported(a))
+  if (g_kernel_family == 0 && tiled_forward_supported(a)) {
+    g_last_family = 2;
     return launch_status(launch_tiled_forward(a, s), "tiled forward launch");
+  }
+  g_last_family = 1;
   return launch_status(launch_general_forward(a, s), "general forward launch");
 }
 
@@ -158,8 +162,11 @@ int backward(void *stream, int reduce, int half_centor, const Dims &d, int group
     a.ref_grad_acc = a.src_grad_acc + ((n_src + 63) / 64) * 64;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (g_kernel_family == 0 && work && tiled_backward_supported(a))
+  if (g_kernel_family == 0 && work && tiled_backward_supported(a)) {
+    g_last_family = 2;
     return launch_status(launch_tiled_backward(a, s), "tiled backward launch");
+  }
+  g_last_family = 1;
   return launch_status(launch_general_backward(a, s), "general backward launch");
 }
 
@@ -179,6 +186,8 @@ int chop_set_kernel_family(int family) {
   g_kernel_family = family == 1 ? 1 : 0;
   return prev;
 }
+
+int chop_last_kernel_family(void) { return g_last_family; }
 
 #define DIMS \
   Dims { B, H, W, C, D, N, srcH, srcW }

@@ -1,0 +1,944 @@
+// Tiled cost-volume kernels for gfx950 (MEAN reduce).
+//
+// Work decomposition.  A workgroup is one wavefront.  It owns PPW = 64/LPP consecutive
+// pixels of one image and one contiguous segment of the D depth hypotheses; the LPP lanes
+// of a pixel each own VEC consecutive channels (C = LPP*VEC), so every tap read and every
+// cost-row write of a pixel is one contiguous C*sizeof(S) segment.  Depth runs innermost:
+// along the walk the sample point of a view slides along an epipolar line by a fraction of
+// a texel per step, so the four bilinear taps of the current texel cell stay in registers
+// and are reloaded only when the cell changes.
+//
+// Each chunk of LPP depths is processed in two phases:
+//   phase 1  lane (pixel p, j) reprojects depth d0+j of pixel p into every view (the
+//            bit-exact code of warp.h), writes the valid-view count and leaves a small
+//            record per (view, depth, pixel) in LDS: tap offset (or -1) and four weights
+//            (backward: also the cell key and four depth-derivative weights);
+//   phase 2  lane (pixel p, channel slice) walks the LPP depths, reading the records as
+//            LDS broadcasts, and does the channel arithmetic with explicit fused
+//            multiply-adds.
+// With LPP == 1 a lane owns its whole pixel and the records stay in registers.
+//
+// Backward keeps, per view, a register image of the source-gradient contributions to the
+// current cell.  When the cell changes the image is added into a per-view LDS
+// window of ROWS x COLS texels that follows the wave's samples along the epipolar lines;
+// neighbouring pixels hit the same texels, so most of the scatter is absorbed there.  A
+// texel reaches memory when the window moves off it, as part of a dense run of
+// global_atomic_add_f32.  ref_grad and the base-plane gradient are pixel-owned and
+// accumulate in registers; they are stored once (one depth segment) or added once per
+// segment.
+#pragma once
+
+#include <type_traits>
+
+#include "internal.h"
+
+namespace chop {
+namespace tiled {
+
+struct Geometry {
+  int hw;                  // H*W
+  int tiles_per_image;     // ceil(hw / PPW)
+  int nseg;                // depth segments
+  int seg;                 // depths per segment, multiple of LPP
+  int64_t total_units;     // B * tiles_per_image * nseg
+  int64_t units_per_xcd;   // ceil(total_units / 8)
+  int sub;                 // channels per correlation group (1 for squared difference)
+};
+
+// ---- vector access ---------------------------------------------------------------------
+template <typename S>
+__device__ __forceinline__ void widen_word(uint32_t w, float *out);
+template <>
+__device__ __forceinline__ void widen_word<float>(uint32_t w, float *out) {
+  out[0] = __uint_as_float(w);
+}
+template <>
+__device__ __forceinline__ void widen_word<__half>(uint32_t w, float *out) {
+  out[0] = __half2float(__ushort_as_half((unsigned short)(w & 0xffffu)));
+  out[1] = __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+}
+template <>
+__device__ __forceinline__ void widen_word<bf16_t>(uint32_t w, float *out) {
+  out[0] = __uint_as_float(w << 16);
+  out[1] = __uint_as_float(w & 0xffff0000u);
+}
+
+template <typename S>
+__device__ __forceinline__ uint32_t narrow_word(const float *in);
+template <>
+__device__ __forceinline__ uint32_t narrow_word<float>(const float *in) {
+  return __float_as_uint(in[0]);
+}
+template <>
+__device__ __forceinline__ uint32_t narrow_word<__half>(const float *in) {
+  return (uint32_t)__half_as_ushort(__float2half_rn(in[0])) |
+         ((uint32_t)__half_as_ushort(__float2half_rn(in[1])) << 16);
+}
+template <>
+__device__ __forceinline__ uint32_t narrow_word<bf16_t>(const float *in) {
+  return float_to_bf16_bits(in[0]) | (float_to_bf16_bits(in[1]) << 16);
+}
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int BYTES>
+struct Raw;
+template <>
+struct Raw<16> {
+  using type = u32x4;
+};
+template <>
+struct Raw<8> {
+  using type = u32x2;
+};
+template <>
+struct Raw<4> {
+  using type = uint32_t;
+};
+template <>
+struct Raw<2> {
+  using type = uint16_t;
+};
+
+// Loads CNT elements of S (CNT*sizeof(S) in {2,4,8,16} bytes, naturally aligned) as floats.
+// STREAM marks data that is touched once (cost rows, upstream gradients): non-temporal.
+template <typename S, int CNT, bool STREAM>
+__device__ __forceinline__ void load_vec(const S *p, float *out) {
+  constexpr int BYTES = CNT * (int)sizeof(S);
+  using RawT = typename Raw<BYTES>::type;
+  constexpr int PER_WORD = 4 / (int)sizeof(S);
+  const RawT *q = reinterpret_cast<const RawT *>(p);
+  const RawT v = STREAM ? __builtin_nontemporal_load(q) : *q;
+  if constexpr (BYTES == 2) {
+    float two[2];
+    widen_word<S>(v, two);
+    out[0] = two[0];
+  } else if constexpr (BYTES == 4) {
+    widen_word<S>(v, out);
+  } else {
+#pragma unroll
+    for (int k = 0; k < BYTES / 4; ++k) widen_word<S>(v[k], out + k * PER_WORD);
+  }
+}
+
+template <typename S, int CNT, bool STREAM>
+__device__ __forceinline__ void store_vec(S *p, const float *in) {
+  constexpr int BYTES = CNT * (int)sizeof(S);
+  using RawT = typename Raw<BYTES>::type;
+  constexpr int PER_WORD = 4 / (int)sizeof(S);
+  RawT *q = reinterpret_cast<RawT *>(p);
+  RawT v;
+  if constexpr (BYTES == 2) {
+    float two[2] = {in[0], 0.f};
+    v = (uint16_t)(narrow_word<S>(two) & 0xffffu);
+  } else if constexpr (BYTES == 4) {
+    v = narrow_word<S>(in);
+  } else {
+#pragma unroll
+    for (int k = 0; k < BYTES / 4; ++k) v[k] = narrow_word<S>(in + k * PER_WORD);
+  }
+  if (STREAM)
+    __builtin_nontemporal_store(v, q);
+  else
+    *q = v;
+}
+
+// Orders this wave's LDS traffic: the lanes of a wavefront execute in lockstep and the
+// LDS returns a wave's operations in issue order, so only the compiler has to be kept
+// from moving accesses across the phase boundary.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int WIDTH>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int m = WIDTH / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, WIDTH);
+  return v;
+}
+
+// Sums the per-channel values of each correlation group: out[g] for g < VEC/sub.
+template <int VEC>
+__device__ __forceinline__ void fold_groups(const float *ch, int sub, float *out) {
+  if (sub == 1) {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) out[c] = ch[c];
+  } else if (sub == 2) {
+#pragma unroll
+    for (int c = 0; c < VEC / 2; ++c) out[c] = ch[2 * c] + ch[2 * c + 1];
+  } else if (sub == 4) {
+#pragma unroll
+    for (int c = 0; c < VEC / 4; ++c)
+      out[c] = (ch[4 * c] + ch[4 * c + 1]) + (ch[4 * c + 2] + ch[4 * c + 3]);
+  } else {  // sub == 8 == VEC
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) s += ch[c];
+    out[0] = s;
+  }
+}
+
+template <typename S, int VEC, bool STREAM>
+__device__ __forceinline__ void store_groups(S *p, const float *v, int sub) {
+  // p already points at this lane's first group
+  if (sub == 1) {
+    store_vec<S, VEC, STREAM>(p, v);
+  } else if (sub == 2) {
+    store_vec<S, VEC / 2, STREAM>(p, v);
+  } else if (sub == 4) {
+    store_vec<S, VEC / 4, STREAM>(p, v);
+  } else {
+    if constexpr (VEC >= 8) store_vec<S, VEC / 8, STREAM>(p, v);
+  }
+}
+
+template <typename S, int VEC, bool STREAM>
+__device__ __forceinline__ void load_groups(const S *p, float *v, int sub) {
+  if (sub == 1) {
+    load_vec<S, VEC, STREAM>(p, v);
+  } else if (sub == 2) {
+    load_vec<S, VEC / 2, STREAM>(p, v);
+  } else if (sub == 4) {
+    load_vec<S, VEC / 4, STREAM>(p, v);
+  } else {
+    if constexpr (VEC >= 8) load_vec<S, VEC / 8, STREAM>(p, v);
+  }
+}
+
+// ---- shared front end of both kernels ---------------------------------------------------
+template <int NV>
+struct Cameras {
+  float zc[NV], wc[NV], hc[NV];  // rows of R applied to (ref_w, ref_h, 1)
+  float t0[NV], t1[NV], t2[NV];
+};
+
+template <int LPP>
+struct Tile {
+  int lane, p, cl;
+  int b, pin, h, w;
+  int d_lo, d_hi;
+  bool pix_ok;
+  int64_t pix;
+};
+
+template <typename S, int LPP>
+__device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g, Tile<LPP> &t) {
+  constexpr int PPW = 64 / LPP;
+  t.lane = threadIdx.x;
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous band
+  // of tiles so that its L2 only has to hold that band's part of the source images.
+  const int64_t bid = blockIdx.x;
+  const int64_t unit = (bid & 7) * g.units_per_xcd + (bid >> 3);
+  if (unit >= g.total_units) return false;
+  const int64_t tile = unit / g.nseg;
+  const int segi = (int)(unit - tile * g.nseg);
+  t.d_lo = segi * g.seg;
+  t.d_hi = min((int)a.D, t.d_lo + g.seg);
+  t.b = (int)(tile / g.tiles_per_image);
+  const int t_in = (int)(tile - (int64_t)t.b * g.tiles_per_image);
+  t.p = t.lane / LPP;
+  t.cl = t.lane % LPP;
+  t.pin = t_in * PPW + t.p;
+  t.pix_ok = t.pin < g.hw;
+  if (!t.pix_ok) t.pin = g.hw - 1;  // clamp: loads stay in range, stores are predicated
+  t.pix = (int64_t)t.b * g.hw + t.pin;
+  t.h = t.pin / (int)a.W;
+  t.w = t.pin - t.h * (int)a.W;
+  return true;
+}
+
+template <typename S, int NV>
+__device__ __forceinline__ void load_cameras(const Args<S> &a, int b, float ref_w, float ref_h,
+                                             Cameras<NV> &c) {
+  const int N = (int)a.N;
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    const int nn = n < N ? n : 0;
+    const float *Rm = a.Rs + ((int64_t)b * N + nn) * 9;
+    const float *t = a.Ts + ((int64_t)b * N + nn) * 3;
+    // same association as the per-voxel expression: (R6*w + R7*h) + R8
+    c.zc[n] = Rm[6] * ref_w + Rm[7] * ref_h + Rm[8];
+    c.wc[n] = Rm[0] * ref_w + Rm[1] * ref_h + Rm[2];
+    c.hc[n] = Rm[3] * ref_w + Rm[4] * ref_h + Rm[5];
+    c.t0[n] = t[0], c.t1[n] = t[1], c.t2[n] = t[2];
+  }
+}
+
+// One reprojection with hoisted row products; bit-identical to warp.h's project().
+struct Hit {
+  int off;     // element offset of tap (fh,fw) inside the view's image, or -1
+  int key;     // (fh << 16) | fw
+  float k00, k01, k11, k10;
+  float dh, dw;
+  float z, w3d, h3d;
+};
+
+template <int NV>
+__device__ __forceinline__ void reproject(const Cameras<NV> &c, int n, float depth, float half,
+                                          int srcH, int srcW, int C, Hit &r) {
+  r.off = -1;
+  r.key = 0;
+  r.k00 = r.k01 = r.k11 = r.k10 = 0.f;
+  r.z = c.zc[n] * depth + c.t2[n];
+  if (r.z <= 0.f) return;
+  r.w3d = c.wc[n] * depth + c.t0[n];
+  float sw = r.w3d / r.z;
+  r.h3d = c.hc[n] * depth + c.t1[n];
+  float sh = r.h3d / r.z;
+  sw = sw - half;
+  sh = sh - half;
+  if (sh > 0.f && sw > 0.f && sh < static_cast<float>(srcH - 1) &&
+      sw < static_cast<float>(srcW - 1)) {
+    const int fh = static_cast<int>(sh), fw = static_cast<int>(sw);
+    r.dh = sh - static_cast<float>(fh);
+    r.dw = sw - static_cast<float>(fw);
+    r.k11 = r.dh * r.dw;
+    r.k10 = r.dh * (1.f - r.dw);
+    r.k00 = (1.f - r.dh) * (1.f - r.dw);
+    r.k01 = (1.f - r.dh) * r.dw;
+    r.off = (fh * srcW + fw) * C;
+    r.key = (fh << 16) | fw;
+  }
+}
+
+template <typename S>
+__device__ __forceinline__ float voxel_depth(const Args<S> &a, int64_t pix, int b, int d,
+                                             float base) {
+  return a.depth_grid ? a.depth_grid[pix * a.D + d] : base + a.offsets[(int64_t)b * a.D + d];
+}
+
+// =========================================================================================
+// Forward
+// =========================================================================================
+template <int NV>
+constexpr int forward_lds_words(int lpp) {
+  return lpp > 1 ? NV * 64 * 5 : 0;
+}
+
+template <typename S, int VEC, int LPP, int NV, int CORR>
+__global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geometry g) {
+  constexpr int PPW = 64 / LPP;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Tile<LPP> t;
+  if (!locate_tile<S, LPP>(a, g, t)) return;
+  const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const float half = a.half;
+  // LDS records: wts[NV][LPP][PPW] then off[NV][LPP][PPW]
+  float4 *s_wts = reinterpret_cast<float4 *>(smem);
+  int *s_off = reinterpret_cast<int *>(s_wts + NV * 64);
+
+  Cameras<NV> cam;
+  load_cameras<S, NV>(a, t.b, static_cast<float>(t.w) + half, static_cast<float>(t.h) + half, cam);
+  const float base = a.depth_grid ? 0.f : a.base_plane[t.pix];
+  float ref[VEC];
+  load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+  const S *view[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n)
+    view[n] = a.src + ((int64_t)t.b * N + (n < N ? n : 0)) * srcH * srcW * C + t.cl * VEC;
+  const int row_step = srcW * C;
+
+  float tap[NV][4][VEC];
+  int cur[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) cur[n] = -1;
+
+  const int OC = CORR ? a.groups : C;
+  const int gv = VEC / g.sub;  // output values per lane
+  const int d_lo = t.d_lo, d_hi = t.d_hi;
+  for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
+    // ---- phase 1: reprojection by lane (p, j = cl) --------------------------------------
+    int r_off[NV];
+    float4 r_wts[NV];
+    {
+      const int d = d0 + t.cl;
+      const bool d_ok = d < d_hi;
+      const float depth = d_ok ? voxel_depth(a, t.pix, t.b, d, base) : 1.f;
+      int cnt = 0;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        Hit hit;
+        hit.off = -1;
+        hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
+        if (n < N && d_ok) reproject<NV>(cam, n, depth, half, srcH, srcW, C, hit);
+        cnt += hit.off >= 0;
+        if constexpr (LPP > 1) {
+          s_off[(n * LPP + t.cl) * PPW + t.p] = hit.off;
+          s_wts[(n * LPP + t.cl) * PPW + t.p] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
+        } else {
+          r_off[n] = hit.off;
+          r_wts[n] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
+        }
+      }
+      if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
+    }
+    if constexpr (LPP > 1) wave_sync();
+    // ---- phase 2: channel arithmetic by lane (p, channel slice) ---------------------------
+#pragma unroll
+    for (int jj = 0; jj < LPP; ++jj) {
+      const int d = d0 + jj;
+      if (d >= d_hi) break;
+      float acc[VEC];
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) acc[c] = 0.f;
+      int k = 0;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        int off;
+        float4 wt;
+        if constexpr (LPP > 1) {
+          off = s_off[(n * LPP + jj) * PPW + t.p];
+          wt = s_wts[(n * LPP + jj) * PPW + t.p];
+        } else {
+          off = r_off[n];
+          wt = r_wts[n];
+        }
+        if (off >= 0) {
+          if (off != cur[n]) {
+            cur[n] = off;
+            const S *q = view[n] + off;
+            load_vec<S, VEC, false>(q, tap[n][0]);
+            load_vec<S, VEC, false>(q + C, tap[n][1]);
+            load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
+            load_vec<S, VEC, false>(q + row_step, tap[n][3]);
+          }
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) {
+            if (CORR == 0) {
+              // sample - ref as one chain of fused multiply-adds
+              float diff = __builtin_fmaf(wt.x, tap[n][0][c], -ref[c]);
+              diff = __builtin_fmaf(wt.y, tap[n][1][c], diff);
+              diff = __builtin_fmaf(wt.z, tap[n][2][c], diff);
+              diff = __builtin_fmaf(wt.w, tap[n][3][c], diff);
+              acc[c] = __builtin_fmaf(diff, diff, acc[c]);
+            } else {
+              float smp = wt.x * tap[n][0][c];
+              smp = __builtin_fmaf(wt.y, tap[n][1][c], smp);
+              smp = __builtin_fmaf(wt.z, tap[n][2][c], smp);
+              smp = __builtin_fmaf(wt.w, tap[n][3][c], smp);
+              acc[c] = __builtin_fmaf(smp, ref[c], acc[c]);
+            }
+          }
+          ++k;
+        }
+      }
+      if (k > 1) {
+        const float inv = __builtin_amdgcn_rcpf(static_cast<float>(k));
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) acc[c] *= inv;
+      }
+      if (t.pix_ok) {
+        S *out = a.cost + (t.pix * D + d) * OC;
+        if (CORR == 0) {
+          store_vec<S, VEC, true>(out + t.cl * VEC, acc);
+        } else {
+          float grp[VEC];
+          fold_groups<VEC>(acc, g.sub, grp);
+          store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
+        }
+      }
+    }
+    if constexpr (LPP > 1) wave_sync();
+  }
+}
+
+// =========================================================================================
+// Backward
+// =========================================================================================
+// Per-view scatter window: a ring buffer of ROWS x COLS texels (C fp32 sums each) addressed
+// by the low bits of the texel coordinates.  `oy, ox` is the window origin: the window
+// holds exactly the texels [oy, oy+ROWS) x [ox, ox+COLS).
+template <int VEC, int LPP>
+struct Window {
+  static constexpr int PPW = 64 / LPP;
+  static constexpr int ROWS = 4;
+  static constexpr int COLS = 2 * PPW > 16 ? 2 * PPW : 16;
+  static constexpr int SLOTS = ROWS * COLS;
+  static constexpr int C = VEC * LPP;
+  static constexpr int STRIDE = C;      // one slot = C consecutive words: 16-byte lane accesses
+  static constexpr int kNone = 0x3fffffff;
+};
+
+template <int VEC, int LPP, int NV>
+constexpr int backward_lds_words() {
+  using WN = Window<VEC, LPP>;
+  // float4 wts, dwt | int off, key | int cnt | float dst | leaving list (slot, texel) | data
+  int w = NV * 64 * 4 * 2 + NV * 64 * 2 + 64 + 64 + WN::SLOTS * 2 + NV * WN::SLOTS * WN::STRIDE;
+  return (w + 3) / 4 * 4;
+}
+
+// Minimum over the 64 lanes, in registers: four DPP steps reduce each row of 16 lanes,
+// four lane reads combine the rows.
+__device__ __forceinline__ int wave_min(int v) {
+  v = min(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false));   // quad_perm 1,0,3,2
+  v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false));   // quad_perm 2,3,0,1
+  v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xf, 0xf, false));  // row_mirror
+  return min(min(__builtin_amdgcn_readlane(v, 0), __builtin_amdgcn_readlane(v, 16)),
+             min(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
+}
+
+// Moves the window of one view to origin (ny, nx): every texel that falls outside the new
+// window is written out with dense global atomics (C consecutive floats per texel, 64/C
+// texels per instruction) and its slot is cleared.  Uniform control flow.
+template <int VEC, int LPP>
+__device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, float *data,
+                                            int *list, float *gview, int srcW, int lane) {
+  using WN = Window<VEC, LPP>;
+  if (oy != WN::kNone) {
+    wave_sync();  // the adds of the chunk before are complete and visible
+    int count = 0;
+    for (int sb = 0; sb < WN::SLOTS; sb += 64) {
+      const int s = sb + lane;
+      const int ry = s / WN::COLS, rx = s % WN::COLS;
+      const int y = oy + ((ry - oy) & (WN::ROWS - 1)), x = ox + ((rx - ox) & (WN::COLS - 1));
+      const bool leaving = !((unsigned)(y - ny) < (unsigned)WN::ROWS &&
+                             (unsigned)(x - nx) < (unsigned)WN::COLS);
+      const unsigned long long m = __ballot(leaving);
+      if (leaving) {
+        const int rank = count + __popcll(m & ((1ull << lane) - 1ull));
+        list[2 * rank] = s;
+        list[2 * rank + 1] = y * srcW + x;
+      }
+      count += __popcll(m);
+    }
+    if (count > 0) {
+      wave_sync();
+      constexpr int EPI = 64 / WN::C;  // texels per instruction
+      const int sub_e = lane / WN::C, j = lane - sub_e * WN::C;
+      for (int e0 = 0; e0 < count; e0 += EPI) {
+        const int e = e0 + sub_e;
+        if (e < count) {
+          float *d = data + list[2 * e] * WN::STRIDE + j;
+          const float v = *d;
+          if (v != 0.f) {
+            *d = 0.f;
+            atomic_add(gview + (int64_t)list[2 * e + 1] * WN::C + j, v);
+          }
+        }
+      }
+      wave_sync();
+    }
+  }
+  oy = ny;
+  ox = nx;
+}
+
+// Adds the four tap images of cell (fh, fw) into the window; taps outside it go to memory.
+// Called from divergent code by all LPP lanes of every pixel whose run just ended.
+// Float LDS atomics cost several cycles per lane, so for wide pixels (LPP >= 4) the window
+// sums are updated with plain 16-byte read-add-write.  Cells of different pixels overlap
+// (a texel is tap 01 of one cell and tap 00 of its neighbour), so the pixels that fire in
+// the same instruction take turns, one pixel per round; usually one or two fire.  Narrow
+// pixels (LPP <= 2: up to 64 pixels per wave) use the atomics instead.
+template <int VEC, int LPP>
+__device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4][VEC],
+                                           float *data, float *gview, int srcW, int lane,
+                                           int cl) {
+  using WN = Window<VEC, LPP>;
+  typedef float vecf __attribute__((ext_vector_type(VEC)));
+  const int fh = key >> 16, fw = key & 0xffff;
+  const int uy = fh - oy, ux = fw - ox;  // >= 0 by construction of the origin
+  const bool in0 = (unsigned)uy < (unsigned)WN::ROWS && (unsigned)ux < (unsigned)WN::COLS;
+  const bool iny1 = (unsigned)(uy + 1) < (unsigned)WN::ROWS;
+  const bool inx1 = (unsigned)(ux + 1) < (unsigned)WN::COLS;
+  const int ry0 = fh & (WN::ROWS - 1), ry1 = (fh + 1) & (WN::ROWS - 1);
+  const int rx0 = fw & (WN::COLS - 1), rx1 = (fw + 1) & (WN::COLS - 1);
+  const int slot[4] = {ry0 * WN::COLS + rx0, ry0 * WN::COLS + rx1, ry1 * WN::COLS + rx1,
+                       ry1 * WN::COLS + rx0};
+  if (in0 && iny1 && inx1) {
+    // the whole cell lies inside the window (the usual case)
+    if constexpr (LPP >= 4) {
+      unsigned long long firing = __ballot(true);
+      while (firing) {
+        const int lead = __ffsll((long long)firing) - 1;
+        firing &= ~(((1ull << LPP) - 1ull) << lead);  // retire this pixel's lanes
+        if (lane - cl == lead) {
+          vecf old[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            old[k] = *reinterpret_cast<vecf *>(data + slot[k] * WN::STRIDE + cl * VEC);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) old[k][i] += v[k][i];
+            *reinterpret_cast<vecf *>(data + slot[k] * WN::STRIDE + cl * VEC) = old[k];
+          }
+        }
+        if (firing) wave_sync();
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        float *d = data + slot[k] * WN::STRIDE + cl * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          __hip_atomic_fetch_add(d + i, v[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      }
+    }
+  } else {
+    // the cell sticks out of the window (samples jumping far apart): add to memory
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int y = fh + (k >> 1), x = fw + ((k == 1 || k == 2) ? 1 : 0);
+      float *gp = gview + (int64_t)(y * srcW + x) * WN::C + cl * VEC;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) atomic_add(gp + i, v[k][i]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[k][i] = 0.f;
+}
+
+template <typename S, int VEC, int LPP, int NV, int CORR>
+__global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geometry g) {
+  using WN = Window<VEC, LPP>;
+  constexpr int PPW = 64 / LPP;
+  constexpr bool kWide = sizeof(S) == 2;  // gradients accumulate in fp32 images
+  extern __shared__ __align__(16) unsigned char smem[];
+  Tile<LPP> t;
+  if (!locate_tile<S, LPP>(a, g, t)) return;
+  const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const float half = a.half;
+  const bool per_voxel_depth = a.depth_grid != nullptr;
+  float4 *s_wts = reinterpret_cast<float4 *>(smem);
+  float4 *s_dwt = s_wts + NV * 64;
+  int *s_off = reinterpret_cast<int *>(s_dwt + NV * 64);
+  int *s_key = s_off + NV * 64;
+  int *s_cnt = s_key + NV * 64;
+  float *s_dst = reinterpret_cast<float *>(s_cnt + 64);
+  int *s_list = reinterpret_cast<int *>(s_dst + 64);
+  float *s_data = reinterpret_cast<float *>(s_list + WN::SLOTS * 2);  // 16-byte aligned
+  for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
+
+  Cameras<NV> cam;
+  load_cameras<S, NV>(a, t.b, static_cast<float>(t.w) + half, static_cast<float>(t.h) + half, cam);
+  const float base = per_voxel_depth ? 0.f : a.base_plane[t.pix];
+  float ref[VEC];
+  load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+  const int64_t view_elems = (int64_t)srcH * srcW * C;
+  float *src_grad_img = kWide ? a.src_grad_acc : reinterpret_cast<float *>(a.src_grad);
+  const S *view[NV];
+  float *gview[NV];  // gradient image of the view, no lane offset
+  int oy[NV], ox[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    const int64_t vo = ((int64_t)t.b * N + (n < N ? n : 0)) * view_elems;
+    view[n] = a.src + vo + t.cl * VEC;
+    gview[n] = src_grad_img + vo;
+    oy[n] = ox[n] = WN::kNone;
+  }
+  const int row_step = srcW * C;
+
+  float tap[NV][4][VEC], sg[NV][4][VEC];
+  int cur[NV], cur_key[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    cur[n] = -1;
+    cur_key[n] = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) sg[n][k][c] = 0.f;
+  }
+  float racc[VEC];
+#pragma unroll
+  for (int c = 0; c < VEC; ++c) racc[c] = 0.f;
+  float dacc = 0.f;  // base-plane gradient partial of this lane
+  wave_sync();
+
+  const int OC = CORR ? a.groups : C;
+  const int gv = VEC / g.sub;
+  const int d_lo = t.d_lo, d_hi = t.d_hi;
+  constexpr int PF = LPP < 8 ? LPP : 8;  // upstream-gradient rows fetched ahead
+  for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
+    int r_off[NV], r_key[NV], r_cnt = 0;
+    float4 r_wts[NV], r_dwt[NV];
+    // The cost_grad rows of this chunk stream from HBM exactly once: issue their loads
+    // now, unconditionally, so that the reprojection below overlaps their latency.
+    float cgr[PF][VEC];
+#pragma unroll
+    for (int jj = 0; jj < PF; ++jj) {
+      const int d = min(d0 + jj, d_hi - 1);
+      const S *src_cg = a.cost_grad + (t.pix * D + d) * OC;
+      if (CORR == 0)
+        load_vec<S, VEC, true>(src_cg + t.cl * VEC, cgr[jj]);
+      else
+        load_groups<S, VEC, true>(src_cg + t.cl * gv, cgr[jj], g.sub);
+    }
+    {
+      const int d = d0 + t.cl;
+      const bool d_ok = d < d_hi;
+      const float depth = d_ok ? voxel_depth(a, t.pix, t.b, d, base) : 1.f;
+      const int cnt = (d_ok && t.pix_ok) ? a.mask_in[t.pix * D + d] : 0;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        Hit hit;
+        hit.off = -1;
+        hit.key = 0;
+        hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
+        float4 dw4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (n < N && cnt > 0) {
+          reproject<NV>(cam, n, depth, half, srcH, srcW, C, hit);
+          if (hit.off >= 0) {
+            // d(sample)/d(depth) = sum over taps of dwt * tap, from
+            //   d/d(src_h) = t1*dw + (t10 - t00),  d/d(src_w) = t1*dh + (t01 - t00),
+            //   t1 = t11 - t10 - t01 + t00, chained through the perspective divide.
+            const float inv = __builtin_amdgcn_rcpf(hit.z * hit.z);
+            const float ah = (cam.hc[n] * hit.z - cam.zc[n] * hit.h3d) * inv;
+            const float aw = (cam.wc[n] * hit.z - cam.zc[n] * hit.w3d) * inv;
+            const float cp = ah * hit.dw + aw * hit.dh;
+            dw4 = make_float4(cp - ah - aw, aw - cp, cp, ah - cp);  // taps 00, 01, 11, 10
+          }
+        }
+        // follow the samples with the scatter window: its origin is the smallest row and
+        // column among this chunk's cells and the cells still open from the last chunk
+        {
+          const bool v1 = hit.off >= 0, v2 = cur[n] >= 0;
+          int my = WN::kNone, mx = WN::kNone;
+          if (v1) my = hit.key >> 16, mx = hit.key & 0xffff;
+          if (v2) my = min(my, cur_key[n] >> 16), mx = min(mx, cur_key[n] & 0xffff);
+          const int ny = wave_min(my), nx = wave_min(mx);
+          if (ny != WN::kNone && (ny != oy[n] || nx != ox[n]))
+            window_move<VEC, LPP>(oy[n], ox[n], ny, nx, s_data + n * WN::SLOTS * WN::STRIDE,
+                                  s_list, gview[n], srcW, t.lane);
+        }
+        if constexpr (LPP > 1) {
+          const int slot = (n * LPP + t.cl) * PPW + t.p;
+          s_off[slot] = hit.off;
+          s_key[slot] = hit.key;
+          s_wts[slot] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
+          s_dwt[slot] = dw4;
+        } else {
+          r_off[n] = hit.off;
+          r_key[n] = hit.key;
+          r_wts[n] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
+          r_dwt[n] = dw4;
+        }
+      }
+      if constexpr (LPP > 1) {
+        s_cnt[t.cl * PPW + t.p] = cnt;
+        s_dst[t.cl * PPW + t.p] = 0.f;
+      } else {
+        r_cnt = cnt;
+      }
+    }
+    if constexpr (LPP > 1) wave_sync();
+#pragma unroll
+    for (int jj = 0; jj < LPP; ++jj) {
+      const int d = d0 + jj;
+      if (d >= d_hi) break;
+      int cnt;
+      if constexpr (LPP > 1)
+        cnt = s_cnt[jj * PPW + t.p];
+      else
+        cnt = r_cnt;
+      if constexpr (LPP > PF) {
+        if (jj == PF) {  // second half of a 16-deep chunk
+#pragma unroll
+          for (int j2 = 0; j2 < PF; ++j2) {
+            const int dd = min(d0 + PF + j2, d_hi - 1);
+            const S *src_cg = a.cost_grad + (t.pix * D + dd) * OC;
+            if (CORR == 0)
+              load_vec<S, VEC, true>(src_cg + t.cl * VEC, cgr[j2]);
+            else
+              load_groups<S, VEC, true>(src_cg + t.cl * gv, cgr[j2], g.sub);
+          }
+        }
+      }
+      // this depth's records, read up front so that their LDS latency overlaps
+      int rec_off[NV];
+      float4 rec_wt[NV], rec_dwt[NV];
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        if constexpr (LPP > 1) {
+          const int slot = (n * LPP + jj) * PPW + t.p;
+          rec_off[n] = s_off[slot];
+          rec_wt[n] = s_wts[slot];
+          rec_dwt[n] = s_dwt[slot];
+        } else {
+          rec_off[n] = r_off[n];
+          rec_wt[n] = r_wts[n];
+          rec_dwt[n] = r_dwt[n];
+        }
+      }
+      float dvox = 0.f;  // this lane's share of d(loss)/d(depth of this voxel)
+      if (cnt > 0) {
+        // upstream gradient per channel, with the factor the reduce applies:
+        // squared difference: 2/k ; correlation: 1/k
+        float cg[VEC];
+        {
+          const float *raw = cgr[jj % PF];
+          if (CORR == 0) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) cg[c] = raw[c];
+          } else {
+            if (g.sub == 1) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) cg[c] = raw[c];
+            } else if (g.sub == 2) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) cg[c] = raw[c / 2];
+            } else if (g.sub == 4) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) cg[c] = raw[c / 4];
+            } else {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) cg[c] = raw[0];
+            }
+          }
+          const float scale =
+              (CORR == 0 ? 2.f : 1.f) * __builtin_amdgcn_rcpf(static_cast<float>(cnt));
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) cg[c] *= scale;
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+          const int off = rec_off[n];
+          const float4 wt = rec_wt[n], dwt = rec_dwt[n];
+          if (off >= 0) {
+            if (off != cur[n]) {
+              // the run on the previous cell ends: hand its image to the window
+              if (cur[n] >= 0)
+                window_add<VEC, LPP>(oy[n], ox[n], cur_key[n], sg[n],
+                                     s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
+                                     t.lane, t.cl);
+              cur[n] = off;
+              if constexpr (LPP > 1)
+                cur_key[n] = s_key[(n * LPP + jj) * PPW + t.p];
+              else
+                cur_key[n] = r_key[n];
+              const S *q = view[n] + off;
+              load_vec<S, VEC, false>(q, tap[n][0]);
+              load_vec<S, VEC, false>(q + C, tap[n][1]);
+              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
+              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
+            }
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+              float gsrc;  // d(loss)/d(sample of this channel)
+              if (CORR == 0) {
+                float diff = __builtin_fmaf(wt.x, tap[n][0][c], -ref[c]);
+                diff = __builtin_fmaf(wt.y, tap[n][1][c], diff);
+                diff = __builtin_fmaf(wt.z, tap[n][2][c], diff);
+                diff = __builtin_fmaf(wt.w, tap[n][3][c], diff);
+                gsrc = diff * cg[c];
+                racc[c] -= gsrc;
+              } else {
+                float smp = wt.x * tap[n][0][c];
+                smp = __builtin_fmaf(wt.y, tap[n][1][c], smp);
+                smp = __builtin_fmaf(wt.z, tap[n][2][c], smp);
+                smp = __builtin_fmaf(wt.w, tap[n][3][c], smp);
+                racc[c] = __builtin_fmaf(cg[c], smp, racc[c]);
+                gsrc = cg[c] * ref[c];
+              }
+              sg[n][0][c] = __builtin_fmaf(gsrc, wt.x, sg[n][0][c]);
+              sg[n][1][c] = __builtin_fmaf(gsrc, wt.y, sg[n][1][c]);
+              sg[n][2][c] = __builtin_fmaf(gsrc, wt.z, sg[n][2][c]);
+              sg[n][3][c] = __builtin_fmaf(gsrc, wt.w, sg[n][3][c]);
+              float ds = dwt.x * tap[n][0][c];
+              ds = __builtin_fmaf(dwt.y, tap[n][1][c], ds);
+              ds = __builtin_fmaf(dwt.z, tap[n][2][c], ds);
+              ds = __builtin_fmaf(dwt.w, tap[n][3][c], ds);
+              dvox = __builtin_fmaf(gsrc, ds, dvox);
+            }
+          }
+        }
+      }
+      if (per_voxel_depth) {
+        if constexpr (LPP > 1) {
+          const float tot = group_sum<LPP>(dvox);
+          if (t.cl == 0) s_dst[jj * PPW + t.p] = tot;
+        } else {
+          if (t.pix_ok) a.depth_grad[t.pix * D + d] = dvox;
+        }
+      } else {
+        dacc += dvox;
+      }
+    }
+    if constexpr (LPP > 1) {
+      wave_sync();
+      if (per_voxel_depth) {
+        const int d = d0 + t.cl;
+        if (d < d_hi && t.pix_ok) a.depth_grad[t.pix * D + d] = s_dst[t.cl * PPW + t.p];
+        wave_sync();
+      }
+    }
+  }
+  // the runs still open, then everything the windows hold
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    if (cur[n] >= 0)
+      window_add<VEC, LPP>(oy[n], ox[n], cur_key[n], sg[n], s_data + n * WN::SLOTS * WN::STRIDE,
+                           gview[n], srcW, t.lane, t.cl);
+  }
+  wave_sync();
+#pragma unroll
+  for (int n = 0; n < NV; ++n)
+    window_move<VEC, LPP>(oy[n], ox[n], -(1 << 20), -(1 << 20),
+                          s_data + n * WN::SLOTS * WN::STRIDE, s_list, gview[n], srcW, t.lane);
+
+  // pixel-owned gradients: one store when this workgroup saw every depth, otherwise one
+  // atomic add per depth segment into the zero-filled outputs
+  float *rg = kWide ? a.ref_grad_acc : reinterpret_cast<float *>(a.ref_grad);
+  if (g.nseg == 1) {
+    if (t.pix_ok) {
+      if (kWide)
+        store_vec<float, VEC, false>(rg + t.pix * C + t.cl * VEC, racc);
+      else
+        store_vec<S, VEC, false>(a.ref_grad + t.pix * C + t.cl * VEC, racc);
+    }
+  } else if (t.pix_ok) {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) atomic_add(rg + t.pix * C + t.cl * VEC + c, racc[c]);
+  }
+  if (!per_voxel_depth) {
+    const float tot = group_sum<LPP>(dacc);
+    if (t.cl == 0 && t.pix_ok) {
+      if (g.nseg == 1)
+        a.depth_grad[t.pix] = tot;
+      else
+        atomic_add(a.depth_grad + t.pix, tot);
+    }
+  }
+}
+
+// ---- host side -------------------------------------------------------------------------------
+// Depth segments: enough workgroups to fill 256 CUs several times over while every segment
+// keeps at least 16 hypotheses for the register-resident taps to pay off.
+inline int choose_segments(int64_t tiles, int64_t D, int lpp) {
+  int nseg = 1;
+  const int64_t min_len = lpp > 16 ? lpp : 16;
+  while (nseg < 8 && tiles * nseg < 256 * 4 * 10 && D / (nseg * 2) >= min_len) nseg *= 2;
+  return nseg;
+}
+
+template <int LPP>
+inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int sub) {
+  constexpr int PPW = 64 / LPP;
+  Geometry g;
+  g.hw = (int)(H * W);
+  g.tiles_per_image = (g.hw + PPW - 1) / PPW;
+  const int64_t tiles = B * g.tiles_per_image;
+  g.nseg = choose_segments(tiles, D, LPP);
+  const int per_seg = (int)((D + g.nseg - 1) / g.nseg);
+  g.seg = ((per_seg + LPP - 1) / LPP) * LPP;
+  g.nseg = (int)((D + g.seg - 1) / g.seg);
+  g.total_units = tiles * g.nseg;
+  g.units_per_xcd = (g.total_units + 7) / 8;
+  g.sub = sub;
+  return g;
+}
+
+template <typename S>
+inline bool aligned16(const S *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+}  // namespace tiled
+}  // namespace chop

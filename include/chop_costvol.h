@@ -184,6 +184,9 @@ int chop_cost_volume_sample_coords_f64(void *stream, int half_centor, int64_t B,
  * (tiled kernels where the shape allows, otherwise the general kernels), 1 = general
  * kernels only.  Returns the previous value.  Used by the tests to cover both. */
 int chop_set_kernel_family(int family);
+/* Which family served the last forward/backward call of this thread: 0 none yet,
+ * 1 general kernels, 2 tiled kernels. */
+int chop_last_kernel_family(void);
 
 #ifdef __cplusplus
 }

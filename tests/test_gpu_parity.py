@@ -23,6 +23,12 @@ def _announce(request):
     _lib.load().chop_set_kernel_family(0)
 
 
+def _assert_family(family, expect_tiled=True):
+    """Under the automatic selection the benchmark shapes must really run the tiled kernels."""
+    got = _lib.load().chop_last_kernel_family()
+    assert got == (1 if family == 1 or not expect_tiled else 2), got
+
+
 def _v1_inputs(t, dtype=None):
     keys = ("ref", "src", "base_plane", "offsets", "Rs", "Ts")
     return [dev(t[k].astype(dtype) if dtype else t[k]) for k in keys]
@@ -95,6 +101,7 @@ def test_v1_forward_tiny_config_full(oracle, family, half):
     want_cost, want_mask = oracle.cost_volume_fwd(t["ref"], t["src"], t["base_plane"], t["offsets"],
                                                   t["Rs"], t["Ts"], "MEAN", half, threads=8)
     cost, mask = chop.cost_volume_raw(*_v1_inputs(t), "MEAN", half)
+    _assert_family(family)
     assert cost.shape == (1, 64, 80, 32, 8) and mask.shape == (1, 64, 80, 32, 1)
     assert np.array_equal(host(mask), want_mask)
     assert_forward_close(host(cost), want_cost)
@@ -111,6 +118,7 @@ def test_v1_forward_benchmark_shapes(oracle, family, index, hw, depth, reduce):
     want_cost, want_mask = oracle.cost_volume_fwd(t["ref"], t["src"], t["base_plane"], t["offsets"],
                                                   t["Rs"], t["Ts"], reduce, threads=8)
     cost, mask = chop.cost_volume_raw(*_v1_inputs(t), reduce)
+    _assert_family(family, expect_tiled=reduce == "MEAN")
     assert np.array_equal(host(mask), want_mask)
     assert_forward_close(host(cost), want_cost)
 
@@ -149,6 +157,7 @@ def test_v1_backward_benchmark_shapes(oracle, family, index, hw, depth):
     _, mask = oracle.cost_volume_fwd(*args, threads=8)
     want = oracle.cost_volume_bwd(*args, t["cost_grad"], mask, threads=1)
     got = chop.cost_volume_grad(*_v1_inputs(t), dev(t["cost_grad"]), dev(mask))
+    _assert_family(family)
     for g, w in zip(got, want):
         assert_backward_close(host(g), w)
     # conservation: ref_grad and src_grad cancel in sum (each g enters as -g and as four
@@ -198,11 +207,13 @@ def test_v2_groupwise_config_f32(oracle, family):
                                                      t["Ts"], "MEAN", 4, threads=8)
     ins = [dev(t[k]) for k in ("ref", "src", "depth_grid", "Rs", "Ts")]
     cost, mask = chop.cost_volume_v2_raw(*ins, "MEAN", 4)
+    _assert_family(family)
     assert np.array_equal(host(mask), want_mask)
     assert_forward_close(host(cost), want_cost, atol=1e-5)
     want = oracle.cost_volume_v2_bwd(t["ref"], t["src"], t["depth_grid"], t["Rs"], t["Ts"],
                                      t["cost_grad"], want_mask, "MEAN", 4)
     got = chop.cost_volume_grad_v2(*ins, dev(t["cost_grad"]), dev(want_mask), "MEAN", 4)
+    _assert_family(family)
     for g, w in zip(got, want):
         assert_backward_close(host(g), w)
 
@@ -229,12 +240,14 @@ def test_v1_16bit_storage(oracle, family, storage):
     ins = [dev(ref, td), dev(src, td), dev(t["base_plane"]), dev(t["offsets"]), dev(t["Rs"]),
            dev(t["Ts"])]
     cost, mask = chop.cost_volume_raw(*ins)
+    _assert_family(family)
     assert cost.dtype == td
     assert np.array_equal(host(mask), want_mask)
     _assert_16bit_close(host(cost), want_cost, storage)
     want = oracle.cost_volume_bwd(ref, src, t["base_plane"], t["offsets"], t["Rs"], t["Ts"], cg,
                                   want_mask)
     got = chop.cost_volume_grad(*ins, dev(cg, td), dev(want_mask))
+    _assert_family(family)
     assert got[0].dtype == td and got[1].dtype == td and got[2].dtype == torch.float32
     for g, w in zip(got, want):
         _assert_16bit_close(host(g), w, storage)
@@ -258,6 +271,7 @@ def test_v2_16bit_storage(oracle, family, storage):
     want = oracle.cost_volume_v2_bwd(ref, src, t["depth_grid"], t["Rs"], t["Ts"], cg, want_mask,
                                      "MEAN", 4)
     got = chop.cost_volume_grad_v2(*ins, dev(cg, td), dev(want_mask), "MEAN", 4)
+    _assert_family(family)
     for g, w in zip(got, want):
         _assert_16bit_close(host(g), w, storage)
 
