@@ -1,0 +1,391 @@
+// TensorFlow-side shim: keeps the op registrations of zhuimeng999/custom_helper_op's
+// cost-volume family and turns each OpKernel into a call of libchop_costvol's C ABI.
+//
+// It is NOT built in this repository's image (no TensorFlow headers exist here); build it
+// where a ROCm TensorFlow is installed:
+//   hipcc/g++ -std=c++17 -shared -fPIC cost_volume_ops.cc -I<repo>/include \
+//       $(python -c 'import tensorflow as tf; print(" ".join(tf.sysconfig.get_compile_flags()))') \
+//       $(python -c 'import tensorflow as tf; print(" ".join(tf.sysconfig.get_link_flags()))') \
+//       -L<repo>/custom_helper_op_amd -lchop_costvol -o _custom_helper_ops.so
+//
+// Drop-in contract (what must not change, with the reference lines that fix it):
+//   op names, input order, attrs, outputs      custom_helper_op/cc/ops/custom_helper_ops.cc:190-307
+//   output shapes [B,H,W,D,C|groups], mask      custom_helper_ops.cc:214-219, :281-286
+//   validation messages and InvalidArgument     cost_volume_kernels.cc:91-106, :220-243;
+//                                               cost_volume_kernels_v2.cc:93-110, :221-247
+//   DEVICE_GPU kernels for float and double     cost_volume_kernels.cc:147-154, :282-289
+//   gradient registered on the Python side      custom_helper_op/python/ops/custom_helper_ops.py:41-96
+// The Python wrapper of the reference loads this library unchanged.
+#define EIGEN_USE_GPU
+
+#include <string>
+
+#include "chop_costvol.h"
+#include "tensorflow/core/framework/op.h"
+#include "tensorflow/core/framework/op_kernel.h"
+#include "tensorflow/core/framework/shape_inference.h"
+
+namespace tensorflow {
+namespace custom_helper_op {
+
+using shape_inference::InferenceContext;
+using shape_inference::ShapeHandle;
+
+namespace {
+
+// cost [B,H,W,D,last], mask [B,H,W,D,1] for MEAN and [B,H,W,D,last] otherwise.
+Status VolumeShapes(InferenceContext* c, int depth_input, int depth_axis, bool grouped) {
+  std::string reduce_method;
+  TF_RETURN_IF_ERROR(c->GetAttr("reduce_method", &reduce_method));
+  ShapeHandle ref, depth;
+  TF_RETURN_IF_ERROR(c->WithRank(c->input(0), 4, &ref));
+  TF_RETURN_IF_ERROR(c->WithRank(c->input(depth_input), depth_axis + 1, &depth));
+  shape_inference::DimensionHandle last = c->Dim(ref, 3);
+  if (grouped) {
+    int32 groups;
+    TF_RETURN_IF_ERROR(c->GetAttr("groups", &groups));
+    last = c->MakeDim(groups);
+  }
+  const auto d = c->Dim(depth, depth_axis);
+  c->set_output(0, c->MakeShape({c->Dim(ref, 0), c->Dim(ref, 1), c->Dim(ref, 2), d, last}));
+  c->set_output(1, c->MakeShape({c->Dim(ref, 0), c->Dim(ref, 1), c->Dim(ref, 2), d,
+                                 reduce_method == "MEAN" ? c->MakeDim(1) : last}));
+  return Status::OK();
+}
+
+Status GradShapes(InferenceContext* c) {
+  for (int i = 0; i < 3; ++i) c->set_output(i, c->input(i));
+  return Status::OK();
+}
+
+}  // namespace
+
+REGISTER_OP("CostVolume")
+    .Input("ref_image: dtype")
+    .Input("src_images: dtype")
+    .Input("base_plane: dtype")
+    .Input("offsets: dtype")
+    .Input("rs: dtype")
+    .Input("ts: dtype")
+    .Attr("dtype: {float32,float64}")
+    .Attr("reduce_method: string")
+    .Attr("half_centor: bool")
+    .Output("cost: dtype")
+    .Output("cost_mask: int32")
+    .SetShapeFn([](InferenceContext* c) { return VolumeShapes(c, 3, 1, false); });
+
+REGISTER_OP("CostVolumeGrad")
+    .Input("ref_image: dtype")
+    .Input("src_images: dtype")
+    .Input("base_plane: dtype")
+    .Input("offsets: dtype")
+    .Input("rs: dtype")
+    .Input("ts: dtype")
+    .Input("cost_grad: dtype")
+    .Input("cost_mask: int32")
+    .Attr("dtype: {float32,float64}")
+    .Attr("reduce_method: string")
+    .Attr("half_centor: bool")
+    .Output("ref_image_grad: dtype")
+    .Output("src_images_grad: dtype")
+    .Output("base_plane_grad: dtype")
+    .SetShapeFn(GradShapes);
+
+REGISTER_OP("CostVolumeV2")
+    .Input("ref_image: dtype")
+    .Input("src_images: dtype")
+    .Input("depth_grid: dtype")
+    .Input("rs: dtype")
+    .Input("ts: dtype")
+    .Attr("dtype: {float32,float64}")
+    .Attr("reduce_method: string")
+    .Attr("groups: int")
+    .Attr("half_centor: bool")
+    .Output("cost: dtype")
+    .Output("cost_mask: int32")
+    .SetShapeFn([](InferenceContext* c) { return VolumeShapes(c, 2, 3, true); });
+
+REGISTER_OP("CostVolumeGradV2")
+    .Input("ref_image: dtype")
+    .Input("src_images: dtype")
+    .Input("depth_grid: dtype")
+    .Input("rs: dtype")
+    .Input("ts: dtype")
+    .Input("cost_grad: dtype")
+    .Input("cost_mask: int32")
+    .Attr("dtype: {float32,float64}")
+    .Attr("reduce_method: string")
+    .Attr("groups: int")
+    .Attr("half_centor: bool")
+    .Output("ref_image_grad: dtype")
+    .Output("src_images_grad: dtype")
+    .Output("base_plane_grad: dtype")
+    .SetShapeFn(GradShapes);
+
+#if GOOGLE_CUDA || TENSORFLOW_USE_ROCM
+
+typedef Eigen::GpuDevice GPUDevice;
+
+namespace {
+
+// One overload set per element type, so the templated kernels below stay type-agnostic.
+inline int Fwd(void* s, int r, int h, const int64* d, const float* a, const float* b,
+               const float* c, const float* e, const float* f, const float* g, float* o,
+               int32* m) {
+  return chop_cost_volume_fwd_f32(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b, c,
+                                  e, f, g, o, m);
+}
+inline int Fwd(void* s, int r, int h, const int64* d, const double* a, const double* b,
+               const double* c, const double* e, const double* f, const double* g, double* o,
+               int32* m) {
+  return chop_cost_volume_fwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b, c,
+                                  e, f, g, o, m);
+}
+inline int Bwd(void* s, int r, int h, const int64* d, const float* a, const float* b,
+               const float* c, const float* e, const float* f, const float* g, const float* cg,
+               const int32* m, float* o0, float* o1, float* o2) {
+  return chop_cost_volume_bwd_f32(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b, c,
+                                  e, f, g, cg, m, o0, o1, o2);
+}
+inline int Bwd(void* s, int r, int h, const int64* d, const double* a, const double* b,
+               const double* c, const double* e, const double* f, const double* g,
+               const double* cg, const int32* m, double* o0, double* o1, double* o2) {
+  return chop_cost_volume_bwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b, c,
+                                  e, f, g, cg, m, o0, o1, o2);
+}
+inline int FwdV2(void* s, int r, int h, const int64* d, int groups, const float* a, const float* b,
+                 const float* c, const float* f, const float* g, float* o, int32* m) {
+  return chop_cost_volume_v2_fwd_f32(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], groups,
+                                     a, b, c, f, g, o, m);
+}
+inline int FwdV2(void* s, int r, int h, const int64* d, int groups, const double* a,
+                 const double* b, const double* c, const double* f, const double* g, double* o,
+                 int32* m) {
+  return chop_cost_volume_v2_fwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], groups,
+                                     a, b, c, f, g, o, m);
+}
+inline int BwdV2(void* s, int r, int h, const int64* d, int groups, const float* a, const float* b,
+                 const float* c, const float* f, const float* g, const float* cg, const int32* m,
+                 float* o0, float* o1, float* o2) {
+  return chop_cost_volume_v2_bwd_f32(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], groups,
+                                     a, b, c, f, g, cg, m, o0, o1, o2);
+}
+inline int BwdV2(void* s, int r, int h, const int64* d, int groups, const double* a,
+                 const double* b, const double* c, const double* f, const double* g,
+                 const double* cg, const int32* m, double* o0, double* o1, double* o2) {
+  return chop_cost_volume_v2_bwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], groups,
+                                     a, b, c, f, g, cg, m, o0, o1, o2);
+}
+
+Status FromChop(int rc) {
+  if (rc == CHOP_OK) return Status::OK();
+  if (rc == CHOP_ERR_LAUNCH || rc == CHOP_ERR_NO_DEVICE)
+    return errors::Internal("libchop_costvol: ", chop_last_error_string());
+  return errors::InvalidArgument("libchop_costvol: ", chop_last_error_string());
+}
+
+// Attributes shared by the four kernels.  An unknown reduce_method is an InvalidArgument
+// at kernel construction (the reference aborts the process with LOG(FATAL),
+// cost_volume_kernels.cc:66-73).
+struct Attrs {
+  int reduce = CHOP_REDUCE_MEAN;
+  bool half_centor = true;
+  int groups = 1;
+  void Read(OpKernelConstruction* ctx, bool grouped) {
+    std::string method;
+    OP_REQUIRES_OK(ctx, ctx->GetAttr("reduce_method", &method));
+    OP_REQUIRES(ctx, method == "MEAN" || method == "MIN",
+                errors::InvalidArgument("Invalid reduce method ", method,
+                                        ". Supported types: MEAN, MIN"));
+    reduce = method == "MEAN" ? CHOP_REDUCE_MEAN : CHOP_REDUCE_MIN;
+    OP_REQUIRES_OK(ctx, ctx->GetAttr("half_centor", &half_centor));
+    if (grouped) OP_REQUIRES_OK(ctx, ctx->GetAttr("groups", &groups));
+  }
+};
+
+// The shape checks of CostVolumeOp::Compute, shared by all four kernels.
+struct Shapes {
+  int64 dims[8];  // B,H,W,C,D,N,srcH,srcW
+  Status Check(const Tensor& ref, const Tensor& src, const Tensor& rs, const Tensor& ts) {
+    if (ref.dims() != 4) return errors::InvalidArgument("ref image must have rank 4");
+    const int64 B = ref.dim_size(0), H = ref.dim_size(1), W = ref.dim_size(2), C = ref.dim_size(3);
+    if (src.dims() != 5 || src.dim_size(0) != B || src.dim_size(2) != H || src.dim_size(3) != W ||
+        src.dim_size(4) != C)
+      return errors::InvalidArgument("src_images must have rank 5, and must compate to ref_image");
+    const int64 N = src.dim_size(1);
+    if (rs.dims() != 4 || rs.dim_size(0) != B || rs.dim_size(1) != N || rs.dim_size(2) != 3 ||
+        rs.dim_size(3) != 3)
+      return errors::InvalidArgument("Rs must have rank 2, and must compate to ref_image");
+    if (ts.dims() != 3 || ts.dim_size(0) != B || ts.dim_size(1) != N || ts.dim_size(2) != 3)
+      return errors::InvalidArgument("Ts must have rank 2, and must compate to ref_image");
+    dims[0] = B, dims[1] = H, dims[2] = W, dims[3] = C, dims[5] = N;
+    dims[6] = src.dim_size(2), dims[7] = src.dim_size(3);
+    return Status::OK();
+  }
+  Status CheckPlane(const Tensor& base_plane, const Tensor& offsets) {
+    if (base_plane.dims() != 4 || base_plane.dim_size(0) != dims[0] ||
+        base_plane.dim_size(1) != dims[1] || base_plane.dim_size(2) != dims[2] ||
+        base_plane.dim_size(3) != 1)
+      return errors::InvalidArgument("base_plane must have rank 4, and must compate to ref_image");
+    if (offsets.dims() != 2 || offsets.dim_size(0) != dims[0])
+      return errors::InvalidArgument("offsets must have rank 2, and must compate to ref_image");
+    dims[4] = offsets.dim_size(1);
+    return Status::OK();
+  }
+  Status CheckGrid(const Tensor& depth_grid, int groups) {
+    if (depth_grid.dims() != 4 || depth_grid.dim_size(0) != dims[0] ||
+        depth_grid.dim_size(1) != dims[1] || depth_grid.dim_size(2) != dims[2])
+      return errors::InvalidArgument("base_plane must have rank 4, and must compate to ref_image");
+    if (groups <= 0 || dims[3] % groups != 0)
+      return errors::InvalidArgument("image_channels and groups_ must match");
+    dims[4] = depth_grid.dim_size(3);
+    return Status::OK();
+  }
+  Status CheckUpstream(const Tensor& cost_grad, const Tensor& cost_mask, int64 last, bool mean) {
+    const TensorShape want({dims[0], dims[1], dims[2], dims[4], last});
+    if (cost_grad.shape() != want)
+      return errors::InvalidArgument("cost_grad must have rank 5, and must compate to ref_image");
+    const TensorShape want_mask({dims[0], dims[1], dims[2], dims[4], mean ? 1 : last});
+    if (cost_mask.shape() != want_mask)
+      return errors::InvalidArgument("cost_mask must have rank 5, and must compate to ref_image");
+    return Status::OK();
+  }
+};
+
+void* StreamOf(OpKernelContext* ctx) {
+  return static_cast<void*>(ctx->eigen_device<GPUDevice>().stream());
+}
+
+}  // namespace
+
+template <typename T>
+class CostVolumeOp : public OpKernel {
+ public:
+  explicit CostVolumeOp(OpKernelConstruction* ctx) : OpKernel(ctx) { attrs_.Read(ctx, false); }
+  void Compute(OpKernelContext* ctx) override {
+    const Tensor &ref = ctx->input(0), &src = ctx->input(1), &plane = ctx->input(2),
+                 &offsets = ctx->input(3), &rs = ctx->input(4), &ts = ctx->input(5);
+    Shapes s;
+    OP_REQUIRES_OK(ctx, s.Check(ref, src, rs, ts));
+    OP_REQUIRES_OK(ctx, s.CheckPlane(plane, offsets));
+    const int64 *d = s.dims;
+    Tensor *cost = nullptr, *mask = nullptr;
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(0, TensorShape({d[0], d[1], d[2], d[4], d[3]}), &cost));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(
+                            1, TensorShape({d[0], d[1], d[2], d[4],
+                                            attrs_.reduce == CHOP_REDUCE_MEAN ? 1 : d[3]}), &mask));
+    OP_REQUIRES_OK(ctx, FromChop(Fwd(StreamOf(ctx), attrs_.reduce, attrs_.half_centor, d,
+                                     ref.flat<T>().data(), src.flat<T>().data(),
+                                     plane.flat<T>().data(), offsets.flat<T>().data(),
+                                     rs.flat<T>().data(), ts.flat<T>().data(),
+                                     cost->flat<T>().data(), mask->flat<int32>().data())));
+  }
+
+ private:
+  Attrs attrs_;
+};
+
+template <typename T>
+class CostVolumeGradOp : public OpKernel {
+ public:
+  explicit CostVolumeGradOp(OpKernelConstruction* ctx) : OpKernel(ctx) { attrs_.Read(ctx, false); }
+  void Compute(OpKernelContext* ctx) override {
+    const Tensor &ref = ctx->input(0), &src = ctx->input(1), &plane = ctx->input(2),
+                 &offsets = ctx->input(3), &rs = ctx->input(4), &ts = ctx->input(5),
+                 &cost_grad = ctx->input(6), &cost_mask = ctx->input(7);
+    Shapes s;
+    OP_REQUIRES_OK(ctx, s.Check(ref, src, rs, ts));
+    OP_REQUIRES_OK(ctx, s.CheckPlane(plane, offsets));
+    OP_REQUIRES_OK(ctx, s.CheckUpstream(cost_grad, cost_mask, s.dims[3],
+                                        attrs_.reduce == CHOP_REDUCE_MEAN));
+    Tensor *g0 = nullptr, *g1 = nullptr, *g2 = nullptr;
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(0, ref.shape(), &g0));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(1, src.shape(), &g1));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(2, plane.shape(), &g2));
+    OP_REQUIRES_OK(ctx, FromChop(Bwd(StreamOf(ctx), attrs_.reduce, attrs_.half_centor, s.dims,
+                                     ref.flat<T>().data(), src.flat<T>().data(),
+                                     plane.flat<T>().data(), offsets.flat<T>().data(),
+                                     rs.flat<T>().data(), ts.flat<T>().data(),
+                                     cost_grad.flat<T>().data(), cost_mask.flat<int32>().data(),
+                                     g0->flat<T>().data(), g1->flat<T>().data(),
+                                     g2->flat<T>().data())));
+  }
+
+ private:
+  Attrs attrs_;
+};
+
+template <typename T>
+class CostVolumeV2Op : public OpKernel {
+ public:
+  explicit CostVolumeV2Op(OpKernelConstruction* ctx) : OpKernel(ctx) { attrs_.Read(ctx, true); }
+  void Compute(OpKernelContext* ctx) override {
+    const Tensor &ref = ctx->input(0), &src = ctx->input(1), &grid = ctx->input(2),
+                 &rs = ctx->input(3), &ts = ctx->input(4);
+    Shapes s;
+    OP_REQUIRES_OK(ctx, s.Check(ref, src, rs, ts));
+    OP_REQUIRES_OK(ctx, s.CheckGrid(grid, attrs_.groups));
+    const int64 *d = s.dims, G = attrs_.groups;
+    Tensor *cost = nullptr, *mask = nullptr;
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(0, TensorShape({d[0], d[1], d[2], d[4], G}), &cost));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(
+                            1, TensorShape({d[0], d[1], d[2], d[4],
+                                            attrs_.reduce == CHOP_REDUCE_MEAN ? 1 : G}), &mask));
+    OP_REQUIRES_OK(ctx, FromChop(FwdV2(StreamOf(ctx), attrs_.reduce, attrs_.half_centor, d,
+                                       attrs_.groups, ref.flat<T>().data(), src.flat<T>().data(),
+                                       grid.flat<T>().data(), rs.flat<T>().data(),
+                                       ts.flat<T>().data(), cost->flat<T>().data(),
+                                       mask->flat<int32>().data())));
+  }
+
+ private:
+  Attrs attrs_;
+};
+
+template <typename T>
+class CostVolumeGradV2Op : public OpKernel {
+ public:
+  explicit CostVolumeGradV2Op(OpKernelConstruction* ctx) : OpKernel(ctx) { attrs_.Read(ctx, true); }
+  void Compute(OpKernelContext* ctx) override {
+    const Tensor &ref = ctx->input(0), &src = ctx->input(1), &grid = ctx->input(2),
+                 &rs = ctx->input(3), &ts = ctx->input(4), &cost_grad = ctx->input(5),
+                 &cost_mask = ctx->input(6);
+    Shapes s;
+    OP_REQUIRES_OK(ctx, s.Check(ref, src, rs, ts));
+    OP_REQUIRES_OK(ctx, s.CheckGrid(grid, attrs_.groups));
+    OP_REQUIRES_OK(ctx, s.CheckUpstream(cost_grad, cost_mask, attrs_.groups,
+                                        attrs_.reduce == CHOP_REDUCE_MEAN));
+    Tensor *g0 = nullptr, *g1 = nullptr, *g2 = nullptr;
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(0, ref.shape(), &g0));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(1, src.shape(), &g1));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(2, grid.shape(), &g2));
+    OP_REQUIRES_OK(ctx, FromChop(BwdV2(StreamOf(ctx), attrs_.reduce, attrs_.half_centor, s.dims,
+                                       attrs_.groups, ref.flat<T>().data(), src.flat<T>().data(),
+                                       grid.flat<T>().data(), rs.flat<T>().data(),
+                                       ts.flat<T>().data(), cost_grad.flat<T>().data(),
+                                       cost_mask.flat<int32>().data(), g0->flat<T>().data(),
+                                       g1->flat<T>().data(), g2->flat<T>().data())));
+  }
+
+ private:
+  Attrs attrs_;
+};
+
+#define REGISTER_CHOP(NAME, CLASS, TYPE) \
+  REGISTER_KERNEL_BUILDER(Name(NAME).Device(DEVICE_GPU).TypeConstraint<TYPE>("dtype"), CLASS<TYPE>)
+
+REGISTER_CHOP("CostVolume", CostVolumeOp, float);
+REGISTER_CHOP("CostVolume", CostVolumeOp, double);
+REGISTER_CHOP("CostVolumeGrad", CostVolumeGradOp, float);
+REGISTER_CHOP("CostVolumeGrad", CostVolumeGradOp, double);
+REGISTER_CHOP("CostVolumeV2", CostVolumeV2Op, float);
+REGISTER_CHOP("CostVolumeV2", CostVolumeV2Op, double);
+REGISTER_CHOP("CostVolumeGradV2", CostVolumeGradV2Op, float);
+REGISTER_CHOP("CostVolumeGradV2", CostVolumeGradV2Op, double);
+
+#undef REGISTER_CHOP
+
+#endif  // GOOGLE_CUDA || TENSORFLOW_USE_ROCM
+
+}  // namespace custom_helper_op
+}  // namespace tensorflow
