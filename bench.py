@@ -158,6 +158,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy, as the known-size reference "
+                         "that HBM traffic counters of a profiler run are scaled by")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this operator runs on one GPU; --gpus %d is not supported "
@@ -173,6 +176,14 @@ def main():
         r.forward()
         r.backward()
     torch.cuda.synchronize()
+    if a.calibrate_copy:
+        n = 256 * 1024 * 1024 // 4
+        src_buf = torch.ones(n, dtype=torch.float32, device="cuda:0")
+        dst_buf = torch.empty_like(src_buf)
+        for _ in range(3):
+            dst_buf.copy_(src_buf)
+        torch.cuda.synchronize()
+        del src_buf, dst_buf
     marks = []
     t0 = time.perf_counter()
     for _ in range(a.steps):
@@ -192,6 +203,13 @@ def main():
     dominant = "backward" if bwd_ms >= fwd_ms else "forward"
     d_ms, d_b = (bwd_ms, bwd_b) if dominant == "backward" else (fwd_ms, fwd_b)
     achieved = d_b / (d_ms * 1e-3) / 1e9
+    traffic = None
+    try:  # measured with rocprofv3 counters in a separate run; the summary is under profiles/
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            t = json.load(f)[wl.name][dominant]
+        traffic = t["fetch_bytes"] + t["write_bytes"]
+    except (OSError, KeyError, ValueError):
+        pass
     out = {
         "metric": "cost-volume voxels/s (B*D*H*W) fwd+bwd",
         "value": wl.voxels / (ms_per_step * 1e-3),
@@ -205,7 +223,7 @@ def main():
             "voxels": wl.voxels, "reduce_method": "MEAN", "half_centor": True},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None,
+                     "traffic": traffic,
                      "algorithmic_bytes": {"forward": fwd_b, "backward": bwd_b},
                      "ms": {"forward": fwd_ms, "backward": bwd_ms},
                      "fwd_bwd_frac": (fwd_b + bwd_b) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS},
