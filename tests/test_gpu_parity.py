@@ -321,3 +321,102 @@ def test_empty_and_degenerate_inputs():
     cmin, mmin = chop.cost_volume_raw(ref, src, torch.ones(1, 4, 5, 1, device="cuda"),
                                       torch.ones(1, 2, device="cuda"), Rs, Ts, "MIN")
     assert bool((mmin == -1).all()) and bool((cmin == torch.finfo(torch.float32).max).all())
+
+
+# ---- committed golden vectors ------------------------------------------------------------------
+@pytest.mark.parametrize("family", FAMILIES)
+def test_golden_vectors(family):
+    """The fixtures of tests/golden/costvol_golden.npz (frozen oracle outputs)."""
+    import os
+    _lib.load().chop_set_kernel_family(family)
+    blob = np.load(os.path.join(os.path.dirname(__file__), "golden", "costvol_golden.npz"))
+    names = sorted({k.split("/")[0] for k in blob.files})
+    for name in names:
+        print("[golden]", name, flush=True)
+        op, red, groups, half = (int(x) for x in blob[name + "/attrs"])
+        t = {k.split("/")[-1]: blob[k] for k in blob.files if k.startswith(name + "/in/")}
+        red_s = "MEAN" if red == 0 else "MIN"
+        want_cost, want_mask = blob[name + "/out/cost"], blob[name + "/out/mask"]
+        if op == 0:
+            ins = [dev(t[k]) for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts")]
+            cost, mask = chop.cost_volume_raw(*ins, red_s, bool(half))
+            got = chop.cost_volume_grad(*ins, dev(t["cost_grad"]), dev(want_mask), red_s, bool(half))
+        else:
+            ins = [dev(t[k]) for k in ("ref", "src", "depth_grid", "Rs", "Ts")]
+            cost, mask = chop.cost_volume_v2_raw(*ins, red_s, groups, bool(half))
+            got = chop.cost_volume_grad_v2(*ins, dev(t["cost_grad"]), dev(want_mask), red_s, groups,
+                                           bool(half))
+        assert np.array_equal(host(mask), want_mask), name
+        if family == 1:
+            assert np.array_equal(host(cost), want_cost), name
+        else:
+            assert_forward_close(host(cost), want_cost, atol=1e-5 if op else 1e-6)
+        tol = 1e-4 if want_cost.dtype == np.float32 else 1e-10
+        for g, k in zip(got, ("ref_grad", "src_grad", "depth_grad")):
+            assert_backward_close(host(g), blob[name + "/out/" + k], tol)
+
+
+# ---- full benchmark sizes -----------------------------------------------------------------------
+def test_mvsnet_stage_full_size(oracle):
+    """Benchmark configuration 2 at its real size, forward and backward, against the oracle
+    (the oracle takes a few seconds on the box's host cores)."""
+    wl = make_workload(2)
+    t = wl.tensors
+    args = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+    want_cost, want_mask = oracle.cost_volume_fwd(*args, threads=16)
+    ins = _v1_inputs(t)
+    cost, mask = chop.cost_volume_raw(*ins)
+    _assert_family(0)
+    assert cost.shape == (1, 128, 160, 192, 32)
+    assert np.array_equal(host(mask), want_mask)
+    assert_forward_close(host(cost), want_cost)
+    del cost
+    want = oracle.cost_volume_bwd(*args, t["cost_grad"], want_mask, threads=16)
+    got = chop.cost_volume_grad(*ins, dev(t["cost_grad"]), mask)
+    _assert_family(0)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+
+
+def test_large_batch_stress_full_size():
+    """Benchmark configuration 5 at its real size (7.25 GB cost volume): size-independent
+    properties on the whole result, the oracle on one band of one batch item."""
+    import oracle
+    wl = make_workload(5, with_cost_grad=False)
+    t = wl.tensors
+    ins = _v1_inputs(t)
+    cost, mask = chop.cost_volume_raw(*ins)
+    _assert_family(0)
+    assert cost.shape == (4, 288, 384, 128, 32) and cost.numel() == 1811939328
+    assert int(mask.min()) >= 0 and int(mask.max()) <= wl.N
+    out_of_frustum = 1.0 - float(mask.float().mean()) / wl.N
+    print("[stress] samples outside every frustum: %.1f%%" % (100 * out_of_frustum), flush=True)
+    assert 0.05 < out_of_frustum < 0.95
+    assert float(cost.min()) >= 0.0
+    assert float((cost.abs() * (mask == 0)).max()) == 0.0  # rows no view reaches stay zero
+    b, r0, r1 = 3, 100, 116
+    band = (t["ref"][b:b + 1, r0:r1], t["src"][b:b + 1], t["base_plane"][b:b + 1, r0:r1],
+            t["offsets"][b:b + 1], t["Rs"][b:b + 1], t["Ts"][b:b + 1])
+    # the oracle runs on reference rows 0..r1 of that batch item (rows above the band are
+    # computed and dropped) so that every pixel keeps its own coordinates
+    want_cost, want_mask = oracle.cost_volume_fwd(
+        t["ref"][b:b + 1, :r1], band[1], t["base_plane"][b:b + 1, :r1], band[3], band[4], band[5],
+        threads=16)
+    got_cost = host(cost[b, r0:r1])
+    got_mask = host(mask[b, r0:r1])
+    assert np.array_equal(got_mask, want_mask[0, r0:r1])
+    assert_forward_close(got_cost, want_cost[0, r0:r1])
+    # backward: linearity in the upstream gradient and conservation, on the full size
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    cg = torch.randn(cost.shape, device="cuda", generator=gen)
+    del cost
+    g1 = chop.cost_volume_grad(*ins, cg, mask)
+    _assert_family(0)
+    rg, sg = g1[0].double(), g1[1].double()
+    assert abs(float(rg.sum() + sg.sum())) < 1e-4 * float(rg.abs().sum())
+    cg.mul_(2.0)
+    g2 = chop.cost_volume_grad(*ins, cg, mask)
+    for a1, a2 in zip(g1, g2):
+        scale = float(a1.abs().max())
+        assert float((a2 - 2 * a1).abs().max()) <= 2e-4 * scale
