@@ -39,8 +39,10 @@ struct Geometry {
   int hw;                  // H*W
   int tiles_per_image;     // ceil(hw / PPW)
   int nseg;                // depth segments
+  int ngroups;             // view groups (backward only): workgroups that split the views
+  int vper;                // views per group
   int seg;                 // depths per segment, multiple of LPP
-  int64_t total_units;     // B * tiles_per_image * nseg
+  int64_t total_units;     // B * tiles_per_image * nseg * ngroups
   int64_t units_per_xcd;   // ceil(total_units / 8)
   int sub;                 // channels per correlation group (1 for squared difference)
 };
@@ -220,6 +222,7 @@ struct Tile {
   int lane, p, cl;
   int b, pin, h, w;
   int d_lo, d_hi;
+  int view0;               // first view of this workgroup's group
   bool pix_ok;
   int64_t pix;
 };
@@ -233,8 +236,13 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
   const int64_t bid = blockIdx.x;
   const int64_t unit = (bid & 7) * g.units_per_xcd + (bid >> 3);
   if (unit >= g.total_units) return false;
-  const int64_t tile = unit / g.nseg;
-  const int segi = (int)(unit - tile * g.nseg);
+  // the groups of one (tile, segment) are neighbours in launch order: they stream the same
+  // upstream-gradient rows at about the same time, through the same L2
+  const int per_tile = g.nseg * g.ngroups;
+  const int64_t tile = unit / per_tile;
+  const int rem = (int)(unit - tile * per_tile);
+  const int segi = rem / g.ngroups;
+  t.view0 = (rem - segi * g.ngroups) * g.vper;
   t.d_lo = segi * g.seg;
   t.d_hi = min((int)a.D, t.d_lo + g.seg);
   t.b = (int)(tile / g.tiles_per_image);
@@ -251,12 +259,12 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
 }
 
 template <typename S, int NV>
-__device__ __forceinline__ void load_cameras(const Args<S> &a, int b, float ref_w, float ref_h,
-                                             Cameras<NV> &c) {
+__device__ __forceinline__ void load_cameras(const Args<S> &a, int b, int view0, float ref_w,
+                                             float ref_h, Cameras<NV> &c) {
   const int N = (int)a.N;
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
-    const int nn = n < N ? n : 0;
+    const int nn = view0 + n < N ? view0 + n : 0;
     const float *Rm = a.Rs + ((int64_t)b * N + nn) * 9;
     const float *t = a.Ts + ((int64_t)b * N + nn) * 3;
     // same association as the per-voxel expression: (R6*w + R7*h) + R8
@@ -331,7 +339,8 @@ __global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geom
   int *s_off = reinterpret_cast<int *>(s_wts + NV * 64);
 
   Cameras<NV> cam;
-  load_cameras<S, NV>(a, t.b, static_cast<float>(t.w) + half, static_cast<float>(t.h) + half, cam);
+  load_cameras<S, NV>(a, t.b, t.view0, static_cast<float>(t.w) + half,
+                      static_cast<float>(t.h) + half, cam);
   const float base = a.depth_grid ? 0.f : a.base_plane[t.pix];
   float ref[VEC];
   load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
@@ -541,7 +550,7 @@ __device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4
   using WN = Window<VEC, LPP>;
   typedef float vecf __attribute__((ext_vector_type(VEC)));
   const int fh = key >> 16, fw = key & 0xffff;
-  const int uy = fh - oy, ux = fw - ox;  // >= 0 by construction of the origin
+  const int uy = fh - oy, ux = fw - ox;
   const bool in0 = (unsigned)uy < (unsigned)WN::ROWS && (unsigned)ux < (unsigned)WN::COLS;
   const bool iny1 = (unsigned)(uy + 1) < (unsigned)WN::ROWS;
   const bool inx1 = (unsigned)(ux + 1) < (unsigned)WN::COLS;
@@ -596,7 +605,7 @@ __device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4
 }
 
 template <typename S, int VEC, int LPP, int NV, int CORR>
-__global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geometry g) {
+__global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const Args<S> a, const Geometry g) {
   using WN = Window<VEC, LPP>;
   constexpr int PPW = 64 / LPP;
   constexpr bool kWide = sizeof(S) == 2;  // gradients accumulate in fp32 images
@@ -617,7 +626,8 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
   for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
 
   Cameras<NV> cam;
-  load_cameras<S, NV>(a, t.b, static_cast<float>(t.w) + half, static_cast<float>(t.h) + half, cam);
+  load_cameras<S, NV>(a, t.b, t.view0, static_cast<float>(t.w) + half,
+                      static_cast<float>(t.h) + half, cam);
   const float base = per_voxel_depth ? 0.f : a.base_plane[t.pix];
   float ref[VEC];
   load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
@@ -628,7 +638,7 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
   int oy[NV], ox[NV];
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
-    const int64_t vo = ((int64_t)t.b * N + (n < N ? n : 0)) * view_elems;
+    const int64_t vo = ((int64_t)t.b * N + (t.view0 + n < N ? t.view0 + n : 0)) * view_elems;
     view[n] = a.src + vo + t.cl * VEC;
     gview[n] = src_grad_img + vo;
     oy[n] = ox[n] = WN::kNone;
@@ -683,7 +693,7 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
         hit.key = 0;
         hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
         float4 dw4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (n < N && cnt > 0) {
+        if (t.view0 + n < N && cnt > 0) {
           reproject<NV>(cam, n, depth, half, srcH, srcW, C, hit);
           if (hit.off >= 0) {
             // d(sample)/d(depth) = sum over taps of dwt * tap, from
@@ -696,17 +706,30 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
             dw4 = make_float4(cp - ah - aw, aw - cp, cp, ah - cp);  // taps 00, 01, 11, 10
           }
         }
-        // follow the samples with the scatter window: its origin is the smallest row and
-        // column among this chunk's cells and the cells still open from the last chunk
+        // follow the samples with the scatter window: it has to cover this chunk's cells and
+        // the cells still open from the last chunk.  It moves only when one of them would
+        // fall outside, and then it is centred on their bounding box.
         {
           const bool v1 = hit.off >= 0, v2 = cur[n] >= 0;
-          int my = WN::kNone, mx = WN::kNone;
-          if (v1) my = hit.key >> 16, mx = hit.key & 0xffff;
-          if (v2) my = min(my, cur_key[n] >> 16), mx = min(mx, cur_key[n] & 0xffff);
+          int my = WN::kNone, mx = WN::kNone, My = -WN::kNone, Mx = -WN::kNone;
+          if (v1) my = My = hit.key >> 16, mx = Mx = hit.key & 0xffff;
+          if (v2) {
+            const int cy = cur_key[n] >> 16, cx = cur_key[n] & 0xffff;
+            my = min(my, cy), mx = min(mx, cx), My = max(My, cy), Mx = max(Mx, cx);
+          }
           const int ny = wave_min(my), nx = wave_min(mx);
-          if (ny != WN::kNone && (ny != oy[n] || nx != ox[n]))
-            window_move<VEC, LPP>(oy[n], ox[n], ny, nx, s_data + n * WN::SLOTS * WN::STRIDE,
-                                  s_list, gview[n], srcW, t.lane);
+          if (ny != WN::kNone) {
+            const int hy = -wave_min(-My) + 1, hx = -wave_min(-Mx) + 1;  // last row / column used
+            const bool fits = oy[n] != WN::kNone && ny >= oy[n] && hy < oy[n] + WN::ROWS &&
+                              nx >= ox[n] && hx < ox[n] + WN::COLS;
+            if (!fits) {
+              const int sy = WN::ROWS - (hy - ny + 1), sx = WN::COLS - (hx - nx + 1);  // slack
+              window_move<VEC, LPP>(oy[n], ox[n], ny - (sy > 0 ? sy / 2 : 0),
+                                    nx - (sx > 0 ? sx / 2 : 0),
+                                    s_data + n * WN::SLOTS * WN::STRIDE, s_list, gview[n], srcW,
+                                    t.lane);
+            }
+          }
         }
         if constexpr (LPP > 1) {
           const int slot = (n * LPP + t.cl) * PPW + t.p;
@@ -729,15 +752,30 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
       }
     }
     if constexpr (LPP > 1) wave_sync();
+    int rb_off[2][NV], rb_cnt[2];
+    float4 rb_wt[2][NV], rb_dwt[2][NV];
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      if constexpr (LPP > 1) {
+        const int slot = (n * LPP) * PPW + t.p;
+        rb_off[0][n] = s_off[slot];
+        rb_wt[0][n] = s_wts[slot];
+        rb_dwt[0][n] = s_dwt[slot];
+      } else {
+        rb_off[0][n] = r_off[n];
+        rb_wt[0][n] = r_wts[n];
+        rb_dwt[0][n] = r_dwt[n];
+      }
+    }
+    if constexpr (LPP > 1)
+      rb_cnt[0] = s_cnt[t.p];
+    else
+      rb_cnt[0] = r_cnt;
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
       if (d >= d_hi) break;
-      int cnt;
-      if constexpr (LPP > 1)
-        cnt = s_cnt[jj * PPW + t.p];
-      else
-        cnt = r_cnt;
+      const int cnt = rb_cnt[jj & 1];
       if constexpr (LPP > PF) {
         if (jj == PF) {  // second half of a 16-deep chunk
 #pragma unroll
@@ -751,22 +789,23 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
           }
         }
       }
-      // this depth's records, read up front so that their LDS latency overlaps
-      int rec_off[NV];
-      float4 rec_wt[NV], rec_dwt[NV];
+      // the records of the NEXT depth are read now, so that their LDS latency overlaps this
+      // depth's arithmetic (jj is unrolled: the buffer index is a compile-time constant)
+      const int cb = jj & 1, nb = cb ^ 1;
+      if constexpr (LPP > 1) {
+        if (jj + 1 < LPP) {
 #pragma unroll
-      for (int n = 0; n < NV; ++n) {
-        if constexpr (LPP > 1) {
-          const int slot = (n * LPP + jj) * PPW + t.p;
-          rec_off[n] = s_off[slot];
-          rec_wt[n] = s_wts[slot];
-          rec_dwt[n] = s_dwt[slot];
-        } else {
-          rec_off[n] = r_off[n];
-          rec_wt[n] = r_wts[n];
-          rec_dwt[n] = r_dwt[n];
+          for (int n = 0; n < NV; ++n) {
+            const int slot = (n * LPP + jj + 1) * PPW + t.p;
+            rb_off[nb][n] = s_off[slot];
+            rb_wt[nb][n] = s_wts[slot];
+            rb_dwt[nb][n] = s_dwt[slot];
+          }
+          rb_cnt[nb] = s_cnt[(jj + 1) * PPW + t.p];
         }
       }
+      const int *rec_off = rb_off[cb];
+      const float4 *rec_wt = rb_wt[cb], *rec_dwt = rb_dwt[cb];
       float dvox = 0.f;  // this lane's share of d(loss)/d(depth of this voxel)
       if (cnt > 0) {
         // upstream gradient per channel, with the factor the reduce applies:
@@ -803,7 +842,13 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
           const float4 wt = rec_wt[n], dwt = rec_dwt[n];
           if (off >= 0) {
             if (off != cur[n]) {
-              // the run on the previous cell ends: hand its image to the window
+              // the run on the previous cell ends.  Start fetching the new cell's taps
+              // first, then hand the old cell's image to the window while they arrive.
+              const S *q = view[n] + off;
+              load_vec<S, VEC, false>(q, tap[n][0]);
+              load_vec<S, VEC, false>(q + C, tap[n][1]);
+              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
+              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
               if (cur[n] >= 0)
                 window_add<VEC, LPP>(oy[n], ox[n], cur_key[n], sg[n],
                                      s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
@@ -813,11 +858,6 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
                 cur_key[n] = s_key[(n * LPP + jj) * PPW + t.p];
               else
                 cur_key[n] = r_key[n];
-              const S *q = view[n] + off;
-              load_vec<S, VEC, false>(q, tap[n][0]);
-              load_vec<S, VEC, false>(q + C, tap[n][1]);
-              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
-              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
             }
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
@@ -855,7 +895,12 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
           const float tot = group_sum<LPP>(dvox);
           if (t.cl == 0) s_dst[jj * PPW + t.p] = tot;
         } else {
-          if (t.pix_ok) a.depth_grad[t.pix * D + d] = dvox;
+          if (t.pix_ok) {
+            if (g.ngroups == 1)
+              a.depth_grad[t.pix * D + d] = dvox;
+            else
+              atomic_add(a.depth_grad + t.pix * D + d, dvox);
+          }
         }
       } else {
         dacc += dvox;
@@ -865,7 +910,12 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
       wave_sync();
       if (per_voxel_depth) {
         const int d = d0 + t.cl;
-        if (d < d_hi && t.pix_ok) a.depth_grad[t.pix * D + d] = s_dst[t.cl * PPW + t.p];
+        if (d < d_hi && t.pix_ok) {
+          if (g.ngroups == 1)
+            a.depth_grad[t.pix * D + d] = s_dst[t.cl * PPW + t.p];
+          else
+            atomic_add(a.depth_grad + t.pix * D + d, s_dst[t.cl * PPW + t.p]);
+        }
         wave_sync();
       }
     }
@@ -886,7 +936,8 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
   // pixel-owned gradients: one store when this workgroup saw every depth, otherwise one
   // atomic add per depth segment into the zero-filled outputs
   float *rg = kWide ? a.ref_grad_acc : reinterpret_cast<float *>(a.ref_grad);
-  if (g.nseg == 1) {
+  const bool single = g.nseg * g.ngroups == 1;
+  if (single) {
     if (t.pix_ok) {
       if (kWide)
         store_vec<float, VEC, false>(rg + t.pix * C + t.cl * VEC, racc);
@@ -900,7 +951,7 @@ __global__ __launch_bounds__(64) void backward_kernel(const Args<S> a, const Geo
   if (!per_voxel_depth) {
     const float tot = group_sum<LPP>(dacc);
     if (t.cl == 0 && t.pix_ok) {
-      if (g.nseg == 1)
+      if (single)
         a.depth_grad[t.pix] = tot;
       else
         atomic_add(a.depth_grad + t.pix, tot);
@@ -919,17 +970,20 @@ inline int choose_segments(int64_t tiles, int64_t D, int lpp) {
 }
 
 template <int LPP>
-inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int sub) {
+inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int sub, int ngroups = 1,
+                              int vper = 0) {
   constexpr int PPW = 64 / LPP;
   Geometry g;
   g.hw = (int)(H * W);
   g.tiles_per_image = (g.hw + PPW - 1) / PPW;
   const int64_t tiles = B * g.tiles_per_image;
-  g.nseg = choose_segments(tiles, D, LPP);
+  g.ngroups = ngroups;
+  g.vper = vper;
+  g.nseg = choose_segments(tiles * ngroups, D, LPP);
   const int per_seg = (int)((D + g.nseg - 1) / g.nseg);
   g.seg = ((per_seg + LPP - 1) / LPP) * LPP;
   g.nseg = (int)((D + g.seg - 1) / g.seg);
-  g.total_units = tiles * g.nseg;
+  g.total_units = tiles * g.nseg * g.ngroups;
   g.units_per_xcd = (g.total_units + 7) / 8;
   g.sub = sub;
   return g;
