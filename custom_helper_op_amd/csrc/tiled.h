@@ -459,7 +459,9 @@ __global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geom
 // =========================================================================================
 // Per-view scatter window: a ring buffer of ROWS x COLS texels (C fp32 sums each) addressed
 // by the low bits of the texel coordinates.  `oy, ox` is the window origin: the window
-// holds exactly the texels [oy, oy+ROWS) x [ox, ox+COLS).
+// holds exactly the texels [oy, oy+ROWS) x [ox, ox+COLS).  Because the slot of a texel
+// depends only on its coordinates, the four slots of a cell are computed once, by the lane
+// that reprojects the voxel, and travel with the record.
 template <int VEC, int LPP>
 struct Window {
   static constexpr int PPW = 64 / LPP;
@@ -469,14 +471,42 @@ struct Window {
   static constexpr int C = VEC * LPP;
   static constexpr int STRIDE = C;      // one slot = C consecutive words: 16-byte lane accesses
   static constexpr int kNone = 0x3fffffff;
+  static constexpr bool kPacked = SLOTS <= 256;  // four slot numbers fit one word
+  static constexpr int kInside = (int)0x80000000u;  // flag in the key word: cell lies in the window
+
+  // slots of the taps 00, 01, 11, 10 of cell `key`, one byte each
+  static __device__ __forceinline__ unsigned pack_slots(int key) {
+    const int fh = (key >> 16) & 0x7fff, fw = key & 0xffff;
+    const int ry0 = (fh & (ROWS - 1)) * COLS, ry1 = ((fh + 1) & (ROWS - 1)) * COLS;
+    const int rx0 = fw & (COLS - 1), rx1 = (fw + 1) & (COLS - 1);
+    return (unsigned)(ry0 + rx0) | ((unsigned)(ry0 + rx1) << 8) | ((unsigned)(ry1 + rx1) << 16) |
+           ((unsigned)(ry1 + rx0) << 24);
+  }
+  // whole cell inside the window at origin (oy, ox)?
+  static __device__ __forceinline__ bool inside(int key, int oy, int ox) {
+    const int fh = (key >> 16) & 0x7fff, fw = key & 0xffff;
+    return (unsigned)(fh - oy) < (unsigned)(ROWS - 1) && (unsigned)(fw - ox) < (unsigned)(COLS - 1);
+  }
 };
 
+// LDS words of the backward kernel: the records of one chunk
+//   float4 wts, dwt [NV*64] | int off [NV*64] | int2 cell {slots, key|inside} [NV*64] |
+//   float scale [64] | float dst [64]
+// then the list of texels leaving a window, then the windows.  With one view per workgroup
+// the list shares the record space: a window only moves before the chunk's records are
+// written.
+template <int VEC, int LPP, int NV>
+constexpr int backward_record_words() {
+  using WN = Window<VEC, LPP>;
+  const int rec = LPP > 1 ? NV * 64 * 11 + 128 : 0;
+  const int list = WN::SLOTS * 2;
+  const int w = NV == 1 ? (rec > list ? rec : list) : rec + list;
+  return (w + 3) / 4 * 4;
+}
 template <int VEC, int LPP, int NV>
 constexpr int backward_lds_words() {
   using WN = Window<VEC, LPP>;
-  // float4 wts, dwt | int off, key | int cnt | float dst | leaving list (slot, texel) | data
-  int w = NV * 64 * 4 * 2 + NV * 64 * 2 + 64 + 64 + WN::SLOTS * 2 + NV * WN::SLOTS * WN::STRIDE;
-  return (w + 3) / 4 * 4;
+  return backward_record_words<VEC, LPP, NV>() + NV * WN::SLOTS * WN::STRIDE;
 }
 
 // Minimum over the 64 lanes, in registers: four DPP steps reduce each row of 16 lanes,
@@ -536,45 +566,47 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
   ox = nx;
 }
 
-// Adds the four tap images of cell (fh, fw) into the window; taps outside it go to memory.
-// Called from divergent code by all LPP lanes of every pixel whose run just ended.
-// Float LDS atomics cost several cycles per lane, so for wide pixels (LPP >= 4) the window
-// sums are updated with plain 16-byte read-add-write.  Cells of different pixels overlap
-// (a texel is tap 01 of one cell and tap 00 of its neighbour), so the pixels that fire in
-// the same instruction take turns, one pixel per round; usually one or two fire.  Narrow
-// pixels (LPP <= 2: up to 64 pixels per wave) use the atomics instead.
+// Adds the four tap images of a finished run into the window; a cell that sticks out of the
+// window goes to memory.  Called from divergent code by all LPP lanes of every pixel whose
+// run just ended.  Float LDS atomics cost several cycles per lane, so for wide pixels
+// (LPP >= 4) the window sums are updated with plain 16-byte read-add-write.  Cells of
+// different pixels overlap (a texel is tap 01 of one cell and tap 00 of its neighbour), so
+// the pixels that fire in the same instruction take turns, one pixel per round; usually one
+// or two fire.  Narrow pixels (LPP <= 2: up to 64 pixels per wave) use the atomics instead.
 template <int VEC, int LPP>
-__device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4][VEC],
+__device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4][VEC],
                                            float *data, float *gview, int srcW, int lane,
                                            int cl) {
   using WN = Window<VEC, LPP>;
   typedef float vecf __attribute__((ext_vector_type(VEC)));
-  const int fh = key >> 16, fw = key & 0xffff;
-  const int uy = fh - oy, ux = fw - ox;
-  const bool in0 = (unsigned)uy < (unsigned)WN::ROWS && (unsigned)ux < (unsigned)WN::COLS;
-  const bool iny1 = (unsigned)(uy + 1) < (unsigned)WN::ROWS;
-  const bool inx1 = (unsigned)(ux + 1) < (unsigned)WN::COLS;
-  const int ry0 = fh & (WN::ROWS - 1), ry1 = (fh + 1) & (WN::ROWS - 1);
-  const int rx0 = fw & (WN::COLS - 1), rx1 = (fw + 1) & (WN::COLS - 1);
-  const int slot[4] = {ry0 * WN::COLS + rx0, ry0 * WN::COLS + rx1, ry1 * WN::COLS + rx1,
-                       ry1 * WN::COLS + rx0};
-  if (in0 && iny1 && inx1) {
+  if (key < 0) {
     // the whole cell lies inside the window (the usual case)
+    if constexpr (!WN::kPacked) slots = 0;
+    int slot[4];
+    if constexpr (WN::kPacked) {
+      slot[0] = slots & 255u, slot[1] = (slots >> 8) & 255u, slot[2] = (slots >> 16) & 255u,
+      slot[3] = slots >> 24;
+    } else {
+      const int fh = (key >> 16) & 0x7fff, fw = key & 0xffff;
+      const int ry0 = (fh & (WN::ROWS - 1)) * WN::COLS, ry1 = ((fh + 1) & (WN::ROWS - 1)) * WN::COLS;
+      const int rx0 = fw & (WN::COLS - 1), rx1 = (fw + 1) & (WN::COLS - 1);
+      slot[0] = ry0 + rx0, slot[1] = ry0 + rx1, slot[2] = ry1 + rx1, slot[3] = ry1 + rx0;
+    }
+    float *base = data + cl * VEC;
     if constexpr (LPP >= 4) {
       unsigned long long firing = __ballot(true);
       while (firing) {
         const int lead = __ffsll((long long)firing) - 1;
         firing &= ~(((1ull << LPP) - 1ull) << lead);  // retire this pixel's lanes
         if (lane - cl == lead) {
-          vecf old[4];
 #pragma unroll
-          for (int k = 0; k < 4; ++k)
-            old[k] = *reinterpret_cast<vecf *>(data + slot[k] * WN::STRIDE + cl * VEC);
+          for (int k0 = 0; k0 < 4; k0 += 2) {
+            vecf o0 = *reinterpret_cast<vecf *>(base + slot[k0] * WN::STRIDE);
+            vecf o1 = *reinterpret_cast<vecf *>(base + slot[k0 + 1] * WN::STRIDE);
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) old[k][i] += v[k][i];
-            *reinterpret_cast<vecf *>(data + slot[k] * WN::STRIDE + cl * VEC) = old[k];
+            for (int i = 0; i < VEC; ++i) o0[i] += v[k0][i], o1[i] += v[k0 + 1][i];
+            *reinterpret_cast<vecf *>(base + slot[k0] * WN::STRIDE) = o0;
+            *reinterpret_cast<vecf *>(base + slot[k0 + 1] * WN::STRIDE) = o1;
           }
         }
         if (firing) wave_sync();
@@ -582,7 +614,7 @@ __device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4
     } else {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
-        float *d = data + slot[k] * WN::STRIDE + cl * VEC;
+        float *d = base + slot[k] * WN::STRIDE;
 #pragma unroll
         for (int i = 0; i < VEC; ++i)
           __hip_atomic_fetch_add(d + i, v[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
@@ -590,6 +622,7 @@ __device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4
     }
   } else {
     // the cell sticks out of the window (samples jumping far apart): add to memory
+    const int fh = key >> 16, fw = key & 0xffff;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int y = fh + (k >> 1), x = fw + ((k == 1 || k == 2) ? 1 : 0);
@@ -604,8 +637,14 @@ __device__ __forceinline__ void window_add(int oy, int ox, int key, float (&v)[4
     for (int i = 0; i < VEC; ++i) v[k][i] = 0.f;
 }
 
+// Waves per SIMD the register budget is held to.  The kernel is latency-bound (its time
+// falls in proportion to the resident waves), so one view per workgroup at three waves
+// beats two views at two.
+constexpr int backward_waves(int nv) { return nv == 1 ? 3 : nv <= 2 ? 2 : 1; }
+
 template <typename S, int VEC, int LPP, int NV, int CORR>
-__global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const Args<S> a, const Geometry g) {
+__global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const Args<S> a,
+                                                                          const Geometry g) {
   using WN = Window<VEC, LPP>;
   constexpr int PPW = 64 / LPP;
   constexpr bool kWide = sizeof(S) == 2;  // gradients accumulate in fp32 images
@@ -617,12 +656,13 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
   const bool per_voxel_depth = a.depth_grid != nullptr;
   float4 *s_wts = reinterpret_cast<float4 *>(smem);
   float4 *s_dwt = s_wts + NV * 64;
-  int *s_off = reinterpret_cast<int *>(s_dwt + NV * 64);
-  int *s_key = s_off + NV * 64;
-  int *s_cnt = s_key + NV * 64;
-  float *s_dst = reinterpret_cast<float *>(s_cnt + 64);
-  int *s_list = reinterpret_cast<int *>(s_dst + 64);
-  float *s_data = reinterpret_cast<float *>(s_list + WN::SLOTS * 2);  // 16-byte aligned
+  int2 *s_cell = reinterpret_cast<int2 *>(s_dwt + NV * 64);
+  int *s_off = reinterpret_cast<int *>(s_cell + NV * 64);
+  float *s_scl = reinterpret_cast<float *>(s_off + NV * 64);
+  float *s_dst = s_scl + 64;
+  int *s_list = NV == 1 ? reinterpret_cast<int *>(smem)
+                        : reinterpret_cast<int *>(smem) + (LPP > 1 ? NV * 64 * 11 + 128 : 0);
+  float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV>();
   for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
 
   Cameras<NV> cam;
@@ -646,11 +686,12 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
   const int row_step = srcW * C;
 
   float tap[NV][4][VEC], sg[NV][4][VEC];
-  int cur[NV], cur_key[NV];
+  int cur[NV];     // tap offset of the open run, -1: none
+  int2 cell[NV];   // its slots and key (bit 31: inside the window)
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
     cur[n] = -1;
-    cur_key[n] = 0;
+    cell[n] = make_int2(0, 0);
 #pragma unroll
     for (int k = 0; k < 4; ++k)
 #pragma unroll
@@ -666,8 +707,11 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   constexpr int PF = LPP < 8 ? LPP : 8;  // upstream-gradient rows fetched ahead
+  const S *cg_lane = a.cost_grad + t.pix * D * OC + t.cl * (CORR ? gv : VEC);
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
-    int r_off[NV], r_key[NV], r_cnt = 0;
+    int r_off[NV];
+    int2 r_cell[NV];
+    float r_scl = 0.f;
     float4 r_wts[NV], r_dwt[NV];
     // The cost_grad rows of this chunk stream from HBM exactly once: issue their loads
     // now, unconditionally, so that the reprojection below overlaps their latency.
@@ -675,17 +719,22 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
 #pragma unroll
     for (int jj = 0; jj < PF; ++jj) {
       const int d = min(d0 + jj, d_hi - 1);
-      const S *src_cg = a.cost_grad + (t.pix * D + d) * OC;
+      const S *src_cg = cg_lane + (int64_t)d * OC;
       if (CORR == 0)
-        load_vec<S, VEC, true>(src_cg + t.cl * VEC, cgr[jj]);
+        load_vec<S, VEC, true>(src_cg, cgr[jj]);
       else
-        load_groups<S, VEC, true>(src_cg + t.cl * gv, cgr[jj], g.sub);
+        load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
     }
     {
       const int d = d0 + t.cl;
       const bool d_ok = d < d_hi;
       const float depth = d_ok ? voxel_depth(a, t.pix, t.b, d, base) : 1.f;
       const int cnt = (d_ok && t.pix_ok) ? a.mask_in[t.pix * D + d] : 0;
+      // factor the reduce applies to the upstream gradient: squared difference 2/k,
+      // correlation 1/k; zero marks a voxel no view saw
+      const float scl = cnt > 0 ? (CORR == 0 ? 2.f : 1.f) *
+                                      __builtin_amdgcn_rcpf(static_cast<float>(cnt))
+                                : 0.f;
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
         Hit hit;
@@ -706,135 +755,108 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
             dw4 = make_float4(cp - ah - aw, aw - cp, cp, ah - cp);  // taps 00, 01, 11, 10
           }
         }
-        // follow the samples with the scatter window: it has to cover this chunk's cells and
-        // the cells still open from the last chunk.  It moves only when one of them would
-        // fall outside, and then it is centred on their bounding box.
-        {
-          const bool v1 = hit.off >= 0, v2 = cur[n] >= 0;
+        // The scatter window has to cover this chunk's cells and the cell still open from
+        // the last chunk.  Usually it already does (one vote); otherwise it is centred on
+        // their bounding box, and whatever still sticks out is marked for the memory path.
+        const bool valid = hit.off >= 0;
+        bool in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
+        if (__ballot(!(in_new && (cur[n] < 0 || cell[n].y < 0))) != 0ull) {
           int my = WN::kNone, mx = WN::kNone, My = -WN::kNone, Mx = -WN::kNone;
-          if (v1) my = My = hit.key >> 16, mx = Mx = hit.key & 0xffff;
-          if (v2) {
-            const int cy = cur_key[n] >> 16, cx = cur_key[n] & 0xffff;
+          if (valid) my = My = hit.key >> 16, mx = Mx = hit.key & 0xffff;
+          if (cur[n] >= 0) {
+            const int cy = (cell[n].y >> 16) & 0x7fff, cx = cell[n].y & 0xffff;
             my = min(my, cy), mx = min(mx, cx), My = max(My, cy), Mx = max(Mx, cx);
           }
           const int ny = wave_min(my), nx = wave_min(mx);
-          if (ny != WN::kNone) {
-            const int hy = -wave_min(-My) + 1, hx = -wave_min(-Mx) + 1;  // last row / column used
-            const bool fits = oy[n] != WN::kNone && ny >= oy[n] && hy < oy[n] + WN::ROWS &&
-                              nx >= ox[n] && hx < ox[n] + WN::COLS;
-            if (!fits) {
-              const int sy = WN::ROWS - (hy - ny + 1), sx = WN::COLS - (hx - nx + 1);  // slack
-              window_move<VEC, LPP>(oy[n], ox[n], ny - (sy > 0 ? sy / 2 : 0),
-                                    nx - (sx > 0 ? sx / 2 : 0),
-                                    s_data + n * WN::SLOTS * WN::STRIDE, s_list, gview[n], srcW,
-                                    t.lane);
-            }
-          }
+          const int hy = -wave_min(-My) + 1, hx = -wave_min(-Mx) + 1;  // last row / column used
+          const int sy = WN::ROWS - (hy - ny + 1), sx = WN::COLS - (hx - nx + 1);  // slack
+          window_move<VEC, LPP>(oy[n], ox[n], ny - (sy > 0 ? sy / 2 : 0),
+                                nx - (sx > 0 ? sx / 2 : 0), s_data + n * WN::SLOTS * WN::STRIDE,
+                                s_list, gview[n], srcW, t.lane);
+          in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
+          const int ck = cell[n].y & 0x7fffffff;
+          cell[n].y = WN::inside(ck, oy[n], ox[n]) ? (ck | WN::kInside) : ck;
         }
+        const int2 rec = make_int2(WN::kPacked ? (int)WN::pack_slots(hit.key) : 0,
+                                   (valid && in_new) ? (hit.key | WN::kInside) : hit.key);
         if constexpr (LPP > 1) {
           const int slot = (n * LPP + t.cl) * PPW + t.p;
           s_off[slot] = hit.off;
-          s_key[slot] = hit.key;
+          s_cell[slot] = rec;
           s_wts[slot] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
           s_dwt[slot] = dw4;
         } else {
           r_off[n] = hit.off;
-          r_key[n] = hit.key;
+          r_cell[n] = rec;
           r_wts[n] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
           r_dwt[n] = dw4;
         }
       }
       if constexpr (LPP > 1) {
-        s_cnt[t.cl * PPW + t.p] = cnt;
+        s_scl[t.cl * PPW + t.p] = scl;
         s_dst[t.cl * PPW + t.p] = 0.f;
       } else {
-        r_cnt = cnt;
+        r_scl = scl;
       }
     }
     if constexpr (LPP > 1) wave_sync();
-    int rb_off[2][NV], rb_cnt[2];
-    float4 rb_wt[2][NV], rb_dwt[2][NV];
-#pragma unroll
-    for (int n = 0; n < NV; ++n) {
-      if constexpr (LPP > 1) {
-        const int slot = (n * LPP) * PPW + t.p;
-        rb_off[0][n] = s_off[slot];
-        rb_wt[0][n] = s_wts[slot];
-        rb_dwt[0][n] = s_dwt[slot];
-      } else {
-        rb_off[0][n] = r_off[n];
-        rb_wt[0][n] = r_wts[n];
-        rb_dwt[0][n] = r_dwt[n];
-      }
-    }
-    if constexpr (LPP > 1)
-      rb_cnt[0] = s_cnt[t.p];
-    else
-      rb_cnt[0] = r_cnt;
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
       if (d >= d_hi) break;
-      const int cnt = rb_cnt[jj & 1];
       if constexpr (LPP > PF) {
         if (jj == PF) {  // second half of a 16-deep chunk
 #pragma unroll
           for (int j2 = 0; j2 < PF; ++j2) {
             const int dd = min(d0 + PF + j2, d_hi - 1);
-            const S *src_cg = a.cost_grad + (t.pix * D + dd) * OC;
+            const S *src_cg = cg_lane + (int64_t)dd * OC;
             if (CORR == 0)
-              load_vec<S, VEC, true>(src_cg + t.cl * VEC, cgr[j2]);
+              load_vec<S, VEC, true>(src_cg, cgr[j2]);
             else
-              load_groups<S, VEC, true>(src_cg + t.cl * gv, cgr[j2], g.sub);
+              load_groups<S, VEC, true>(src_cg, cgr[j2], g.sub);
           }
         }
       }
-      // the records of the NEXT depth are read now, so that their LDS latency overlaps this
-      // depth's arithmetic (jj is unrolled: the buffer index is a compile-time constant)
-      const int cb = jj & 1, nb = cb ^ 1;
+      // this depth's records (LDS broadcasts); the other waves of the SIMD cover the latency
+      int rec_off[NV];
+      float4 rec_wt[NV], rec_dwt[NV];
+      float scl;
       if constexpr (LPP > 1) {
-        if (jj + 1 < LPP) {
 #pragma unroll
-          for (int n = 0; n < NV; ++n) {
-            const int slot = (n * LPP + jj + 1) * PPW + t.p;
-            rb_off[nb][n] = s_off[slot];
-            rb_wt[nb][n] = s_wts[slot];
-            rb_dwt[nb][n] = s_dwt[slot];
-          }
-          rb_cnt[nb] = s_cnt[(jj + 1) * PPW + t.p];
+        for (int n = 0; n < NV; ++n) {
+          const int slot = (n * LPP + jj) * PPW + t.p;
+          rec_off[n] = s_off[slot];
+          rec_wt[n] = s_wts[slot];
+          rec_dwt[n] = s_dwt[slot];
         }
+        scl = s_scl[jj * PPW + t.p];
+      } else {
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+          rec_off[n] = r_off[n];
+          rec_wt[n] = r_wts[n];
+          rec_dwt[n] = r_dwt[n];
+        }
+        scl = r_scl;
       }
-      const int *rec_off = rb_off[cb];
-      const float4 *rec_wt = rb_wt[cb], *rec_dwt = rb_dwt[cb];
       float dvox = 0.f;  // this lane's share of d(loss)/d(depth of this voxel)
-      if (cnt > 0) {
-        // upstream gradient per channel, with the factor the reduce applies:
-        // squared difference: 2/k ; correlation: 1/k
+      if (scl != 0.f) {
         float cg[VEC];
         {
           const float *raw = cgr[jj % PF];
-          if (CORR == 0) {
+          if (CORR == 0 || g.sub == 1) {
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) cg[c] = raw[c];
+            for (int c = 0; c < VEC; ++c) cg[c] = raw[c] * scl;
+          } else if (g.sub == 2) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) cg[c] = raw[c / 2] * scl;
+          } else if (g.sub == 4) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) cg[c] = raw[c / 4] * scl;
           } else {
-            if (g.sub == 1) {
 #pragma unroll
-              for (int c = 0; c < VEC; ++c) cg[c] = raw[c];
-            } else if (g.sub == 2) {
-#pragma unroll
-              for (int c = 0; c < VEC; ++c) cg[c] = raw[c / 2];
-            } else if (g.sub == 4) {
-#pragma unroll
-              for (int c = 0; c < VEC; ++c) cg[c] = raw[c / 4];
-            } else {
-#pragma unroll
-              for (int c = 0; c < VEC; ++c) cg[c] = raw[0];
-            }
+            for (int c = 0; c < VEC; ++c) cg[c] = raw[0] * scl;
           }
-          const float scale =
-              (CORR == 0 ? 2.f : 1.f) * __builtin_amdgcn_rcpf(static_cast<float>(cnt));
-#pragma unroll
-          for (int c = 0; c < VEC; ++c) cg[c] *= scale;
         }
 #pragma unroll
         for (int n = 0; n < NV; ++n) {
@@ -850,14 +872,14 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
               load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
               load_vec<S, VEC, false>(q + row_step, tap[n][3]);
               if (cur[n] >= 0)
-                window_add<VEC, LPP>(oy[n], ox[n], cur_key[n], sg[n],
+                window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
                                      s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
                                      t.lane, t.cl);
               cur[n] = off;
               if constexpr (LPP > 1)
-                cur_key[n] = s_key[(n * LPP + jj) * PPW + t.p];
+                cell[n] = s_cell[(n * LPP + jj) * PPW + t.p];
               else
-                cur_key[n] = r_key[n];
+                cell[n] = r_cell[n];
             }
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
@@ -924,8 +946,8 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
     if (cur[n] >= 0)
-      window_add<VEC, LPP>(oy[n], ox[n], cur_key[n], sg[n], s_data + n * WN::SLOTS * WN::STRIDE,
-                           gview[n], srcW, t.lane, t.cl);
+      window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
+                           s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW, t.lane, t.cl);
   }
   wave_sync();
 #pragma unroll
@@ -962,10 +984,10 @@ __global__ __launch_bounds__(64, (NV <= 2 ? 2 : 1)) void backward_kernel(const A
 // ---- host side -------------------------------------------------------------------------------
 // Depth segments: enough workgroups to fill 256 CUs several times over while every segment
 // keeps at least 16 hypotheses for the register-resident taps to pay off.
-inline int choose_segments(int64_t tiles, int64_t D, int lpp) {
+inline int choose_segments(int64_t tiles, int64_t D, int lpp, int64_t target_units) {
   int nseg = 1;
   const int64_t min_len = lpp > 16 ? lpp : 16;
-  while (nseg < 8 && tiles * nseg < 256 * 4 * 10 && D / (nseg * 2) >= min_len) nseg *= 2;
+  while (nseg < 8 && tiles * nseg < target_units && D / (nseg * 2) >= min_len) nseg *= 2;
   return nseg;
 }
 
@@ -979,7 +1001,8 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   const int64_t tiles = B * g.tiles_per_image;
   g.ngroups = ngroups;
   g.vper = vper;
-  g.nseg = choose_segments(tiles * ngroups, D, LPP);
+  // the backward kernel (the one with view groups) runs more, lighter waves per CU
+  g.nseg = choose_segments(tiles * ngroups, D, LPP, vper > 0 ? 256 * 4 * 20 : 256 * 4 * 10);
   const int per_seg = (int)((D + g.nseg - 1) / g.nseg);
   g.seg = ((per_seg + LPP - 1) / LPP) * LPP;
   g.nseg = (int)((D + g.seg - 1) / g.seg);
