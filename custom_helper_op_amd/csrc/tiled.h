@@ -149,6 +149,12 @@ __device__ __forceinline__ void store_vec(S *p, const float *in) {
 // Orders this wave's LDS traffic: the lanes of a wavefront execute in lockstep and the
 // LDS returns a wave's operations in issue order, so only the compiler has to be kept
 // from moving accesses across the phase boundary.
+// An LDS object at (lane-dependent byte offset) + (compile-time constant).
+template <typename T>
+__device__ __forceinline__ T &lds_at(unsigned char *base, unsigned lane_bytes, int const_bytes) {
+  return *reinterpret_cast<T *>(base + lane_bytes + const_bytes);
+}
+
 __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -334,9 +340,12 @@ __global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geom
   if (!locate_tile<S, LPP>(a, g, t)) return;
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
   const float half = a.half;
-  // LDS records: wts[NV][LPP][PPW] then off[NV][LPP][PPW]
-  float4 *s_wts = reinterpret_cast<float4 *>(smem);
-  int *s_off = reinterpret_cast<int *>(s_wts + NV * 64);
+  // LDS records: wts[NV][LPP][PPW] then off[NV][LPP][PPW], addressed as (lane-dependent
+  // byte offset) + (compile-time constant) so that the constant lands in the instruction's
+  // offset field instead of costing a register per unrolled depth
+  constexpr int kWts = 0, kOff = NV * 64 * 16;
+  const unsigned p4 = (unsigned)t.p * 4u;                 // reader: pixel p
+  const unsigned q4 = (unsigned)(t.cl * PPW + t.p) * 4u;  // writer: lane (p, j)
 
   Cameras<NV> cam;
   load_cameras<S, NV>(a, t.b, t.view0, static_cast<float>(t.w) + half,
@@ -375,8 +384,9 @@ __global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geom
         if (n < N && d_ok) reproject<NV>(cam, n, depth, half, srcH, srcW, C, hit);
         cnt += hit.off >= 0;
         if constexpr (LPP > 1) {
-          s_off[(n * LPP + t.cl) * PPW + t.p] = hit.off;
-          s_wts[(n * LPP + t.cl) * PPW + t.p] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
+          lds_at<int>(smem, q4, kOff + (n * LPP * PPW) * 4) = hit.off;
+          lds_at<float4>(smem, q4 * 4u, kWts + (n * LPP * PPW) * 16) =
+              make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
         } else {
           r_off[n] = hit.off;
           r_wts[n] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
@@ -399,8 +409,8 @@ __global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geom
         int off;
         float4 wt;
         if constexpr (LPP > 1) {
-          off = s_off[(n * LPP + jj) * PPW + t.p];
-          wt = s_wts[(n * LPP + jj) * PPW + t.p];
+          off = lds_at<int>(smem, p4, kOff + ((n * LPP + jj) * PPW) * 4);
+          wt = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj) * PPW) * 16);
         } else {
           off = r_off[n];
           wt = r_wts[n];
@@ -640,10 +650,10 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
 // Waves per SIMD the register budget is held to.  The kernel is latency-bound (its time
 // falls in proportion to the resident waves), so one view per workgroup at three waves
 // beats two views at two.
-constexpr int backward_waves(int nv) { return nv == 1 ? 3 : nv <= 2 ? 2 : 1; }
+constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 : nv <= 2 ? 2 : 1; }
 
 template <typename S, int VEC, int LPP, int NV, int CORR>
-__global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const Args<S> a,
+__global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
   using WN = Window<VEC, LPP>;
   constexpr int PPW = 64 / LPP;
@@ -654,12 +664,12 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
   const float half = a.half;
   const bool per_voxel_depth = a.depth_grid != nullptr;
-  float4 *s_wts = reinterpret_cast<float4 *>(smem);
-  float4 *s_dwt = s_wts + NV * 64;
-  int2 *s_cell = reinterpret_cast<int2 *>(s_dwt + NV * 64);
-  int *s_off = reinterpret_cast<int *>(s_cell + NV * 64);
-  float *s_scl = reinterpret_cast<float *>(s_off + NV * 64);
-  float *s_dst = s_scl + 64;
+  // byte offsets of the record arrays; a record is addressed as (lane-dependent byte offset)
+  // + (compile-time constant), so that the constant lands in the instruction's offset field
+  constexpr int kWts = 0, kDwt = kWts + NV * 64 * 16, kCell = kDwt + NV * 64 * 16,
+                kOff = kCell + NV * 64 * 8, kScl = kOff + NV * 64 * 4, kDst = kScl + 64 * 4;
+  const unsigned p4 = (unsigned)t.p * 4u;                      // reader: pixel p
+  const unsigned q4 = (unsigned)(t.cl * PPW + t.p) * 4u;       // writer: lane (p, j)
   int *s_list = NV == 1 ? reinterpret_cast<int *>(smem)
                         : reinterpret_cast<int *>(smem) + (LPP > 1 ? NV * 64 * 11 + 128 : 0);
   float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV>();
@@ -708,7 +718,18 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   constexpr int PF = LPP < 8 ? LPP : 8;  // upstream-gradient rows fetched ahead
   const S *cg_lane = a.cost_grad + t.pix * D * OC + t.cl * (CORR ? gv : VEC);
+  const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
+  const int32_t *cnt_src = a.mask_in + t.pix * D;
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
+    // Depth hypothesis and valid-view count of lane (p, j)'s voxel: requested before the
+    // chunk's upstream-gradient rows, because loads return in order and the reprojection
+    // should wait for these two words only.
+    float dv = 1.f;
+    int cnt = 0;
+    if (d0 + t.cl < d_hi) {
+      dv = dv_src[d0 + t.cl];
+      if (t.pix_ok) cnt = cnt_src[d0 + t.cl];
+    }
     int r_off[NV];
     int2 r_cell[NV];
     float r_scl = 0.f;
@@ -726,10 +747,7 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
         load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
     }
     {
-      const int d = d0 + t.cl;
-      const bool d_ok = d < d_hi;
-      const float depth = d_ok ? voxel_depth(a, t.pix, t.b, d, base) : 1.f;
-      const int cnt = (d_ok && t.pix_ok) ? a.mask_in[t.pix * D + d] : 0;
+      const float depth = d0 + t.cl < d_hi ? (per_voxel_depth ? dv : base + dv) : 1.f;
       // factor the reduce applies to the upstream gradient: squared difference 2/k,
       // correlation 1/k; zero marks a voxel no view saw
       const float scl = cnt > 0 ? (CORR == 0 ? 2.f : 1.f) *
@@ -780,11 +798,11 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
         const int2 rec = make_int2(WN::kPacked ? (int)WN::pack_slots(hit.key) : 0,
                                    (valid && in_new) ? (hit.key | WN::kInside) : hit.key);
         if constexpr (LPP > 1) {
-          const int slot = (n * LPP + t.cl) * PPW + t.p;
-          s_off[slot] = hit.off;
-          s_cell[slot] = rec;
-          s_wts[slot] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
-          s_dwt[slot] = dw4;
+          lds_at<int>(smem, q4, kOff + (n * LPP * PPW) * 4) = hit.off;
+          lds_at<int2>(smem, q4 * 2u, kCell + (n * LPP * PPW) * 8) = rec;
+          lds_at<float4>(smem, q4 * 4u, kWts + (n * LPP * PPW) * 16) =
+              make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
+          lds_at<float4>(smem, q4 * 4u, kDwt + (n * LPP * PPW) * 16) = dw4;
         } else {
           r_off[n] = hit.off;
           r_cell[n] = rec;
@@ -793,8 +811,8 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
         }
       }
       if constexpr (LPP > 1) {
-        s_scl[t.cl * PPW + t.p] = scl;
-        s_dst[t.cl * PPW + t.p] = 0.f;
+        lds_at<float>(smem, q4, kScl) = scl;
+        lds_at<float>(smem, q4, kDst) = 0.f;
       } else {
         r_scl = scl;
       }
@@ -824,12 +842,11 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
       if constexpr (LPP > 1) {
 #pragma unroll
         for (int n = 0; n < NV; ++n) {
-          const int slot = (n * LPP + jj) * PPW + t.p;
-          rec_off[n] = s_off[slot];
-          rec_wt[n] = s_wts[slot];
-          rec_dwt[n] = s_dwt[slot];
+          rec_off[n] = lds_at<int>(smem, p4, kOff + ((n * LPP + jj) * PPW) * 4);
+          rec_wt[n] = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj) * PPW) * 16);
+          rec_dwt[n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj) * PPW) * 16);
         }
-        scl = s_scl[jj * PPW + t.p];
+        scl = lds_at<float>(smem, p4, kScl + (jj * PPW) * 4);
       } else {
 #pragma unroll
         for (int n = 0; n < NV; ++n) {
@@ -877,7 +894,7 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
                                      t.lane, t.cl);
               cur[n] = off;
               if constexpr (LPP > 1)
-                cell[n] = s_cell[(n * LPP + jj) * PPW + t.p];
+                cell[n] = lds_at<int2>(smem, p4 * 2u, kCell + ((n * LPP + jj) * PPW) * 8);
               else
                 cell[n] = r_cell[n];
             }
@@ -915,7 +932,7 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
       if (per_voxel_depth) {
         if constexpr (LPP > 1) {
           const float tot = group_sum<LPP>(dvox);
-          if (t.cl == 0) s_dst[jj * PPW + t.p] = tot;
+          if (t.cl == 0) lds_at<float>(smem, p4, kDst + (jj * PPW) * 4) = tot;
         } else {
           if (t.pix_ok) {
             if (g.ngroups == 1)
@@ -934,9 +951,9 @@ __global__ __launch_bounds__(64, backward_waves(NV)) void backward_kernel(const 
         const int d = d0 + t.cl;
         if (d < d_hi && t.pix_ok) {
           if (g.ngroups == 1)
-            a.depth_grad[t.pix * D + d] = s_dst[t.cl * PPW + t.p];
+            a.depth_grad[t.pix * D + d] = lds_at<float>(smem, q4, kDst);
           else
-            atomic_add(a.depth_grad + t.pix * D + d, s_dst[t.cl * PPW + t.p]);
+            atomic_add(a.depth_grad + t.pix * D + d, lds_at<float>(smem, q4, kDst));
         }
         wave_sync();
       }
