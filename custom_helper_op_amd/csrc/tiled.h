@@ -44,6 +44,8 @@ struct Geometry {
   int seg;                 // depths per segment, multiple of LPP
   int64_t total_units;     // B * tiles_per_image * nseg * ngroups
   int64_t units_per_xcd;   // ceil(total_units / 8)
+  int xcd_run;             // consecutive units dealt to one XCD at a time
+  int64_t grid;            // workgroups to launch
   int sub;                 // channels per correlation group (1 for squared difference)
 };
 
@@ -237,10 +239,13 @@ template <typename S, int LPP>
 __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g, Tile<LPP> &t) {
   constexpr int PPW = 64 / LPP;
   t.lane = threadIdx.x;
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous band
-  // of tiles so that its L2 only has to hold that band's part of the source images.
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD runs of consecutive
+  // tiles so that its L2 only has to hold that part of the source images.  Forward: one
+  // band per XCD.  Backward: short runs, which balance the XCDs better (its tiles differ
+  // more in cost).
   const int64_t bid = blockIdx.x;
-  const int64_t unit = (bid & 7) * g.units_per_xcd + (bid >> 3);
+  const int64_t r = bid >> 3;
+  const int64_t unit = (r / g.xcd_run) * (8 * (int64_t)g.xcd_run) + (bid & 7) * g.xcd_run + r % g.xcd_run;
   if (unit >= g.total_units) return false;
   // the groups of one (tile, segment) are neighbours in launch order: they stream the same
   // upstream-gradient rows at about the same time, through the same L2
@@ -734,17 +739,19 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     int2 r_cell[NV];
     float r_scl = 0.f;
     float4 r_wts[NV], r_dwt[NV];
-    // The cost_grad rows of this chunk stream from HBM exactly once: issue their loads
-    // now, unconditionally, so that the reprojection below overlaps their latency.
+    // Issue the loads of this chunk's cost_grad rows now, unconditionally, so that the
+    // reprojection below overlaps their latency.  They are ordinary (cached) loads: the
+    // workgroup of the next view reads the same rows a moment later and should find them
+    // in L2.
     float cgr[PF][VEC];
 #pragma unroll
     for (int jj = 0; jj < PF; ++jj) {
       const int d = min(d0 + jj, d_hi - 1);
       const S *src_cg = cg_lane + (int64_t)d * OC;
       if (CORR == 0)
-        load_vec<S, VEC, true>(src_cg, cgr[jj]);
+        load_vec<S, VEC, false>(src_cg, cgr[jj]);
       else
-        load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
+        load_groups<S, VEC, false>(src_cg, cgr[jj], g.sub);
     }
     {
       const float depth = d0 + t.cl < d_hi ? (per_voxel_depth ? dv : base + dv) : 1.f;
@@ -829,9 +836,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
             const int dd = min(d0 + PF + j2, d_hi - 1);
             const S *src_cg = cg_lane + (int64_t)dd * OC;
             if (CORR == 0)
-              load_vec<S, VEC, true>(src_cg, cgr[j2]);
+              load_vec<S, VEC, false>(src_cg, cgr[j2]);
             else
-              load_groups<S, VEC, true>(src_cg, cgr[j2], g.sub);
+              load_groups<S, VEC, false>(src_cg, cgr[j2], g.sub);
           }
         }
       }
@@ -1025,6 +1032,11 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   g.nseg = (int)((D + g.seg - 1) / g.seg);
   g.total_units = tiles * g.nseg * g.ngroups;
   g.units_per_xcd = (g.total_units + 7) / 8;
+  // backward: about 32 units per run, whole pixel tiles (their view groups share L2 lines)
+  const int per_tile = g.nseg * g.ngroups;
+  g.xcd_run = vper > 0 ? per_tile * (32 / per_tile > 1 ? 32 / per_tile : 1)
+                       : (int)(g.units_per_xcd > 0 ? g.units_per_xcd : 1);
+  g.grid = (g.total_units + 8 * (int64_t)g.xcd_run - 1) / (8 * (int64_t)g.xcd_run) * (8 * (int64_t)g.xcd_run);
   g.sub = sub;
   return g;
 }
