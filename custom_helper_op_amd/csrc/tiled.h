@@ -44,7 +44,7 @@ struct Geometry {
   int seg;                 // depths per segment, multiple of LPP
   int64_t total_units;     // B * tiles_per_image * nseg * ngroups
   int64_t units_per_xcd;   // ceil(total_units / 8)
-  int xcd_run;             // consecutive units dealt to one XCD at a time
+  int xcd_shift;           // log2 of the units dealt to one XCD at a time; -1: one band per XCD
   int64_t grid;            // workgroups to launch
   int sub;                 // channels per correlation group (1 for squared difference)
 };
@@ -243,21 +243,26 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
   // tiles so that its L2 only has to hold that part of the source images.  Forward: one
   // band per XCD.  Backward: short runs, which balance the XCDs better (its tiles differ
   // more in cost).
-  const int64_t bid = blockIdx.x;
-  const int64_t r = bid >> 3;
-  const int64_t unit = (r / g.xcd_run) * (8 * (int64_t)g.xcd_run) + (bid & 7) * g.xcd_run + r % g.xcd_run;
-  if (unit >= g.total_units) return false;
+  // (all counts fit 32 bits: the host checks total_units; 64-bit divisions would cost
+  // several hundred instructions per workgroup, which runs only a few thousand)
+  const unsigned bid = blockIdx.x;
+  const unsigned r = bid >> 3, x = bid & 7u;
+  const unsigned unit = g.xcd_shift < 0
+                            ? x * (unsigned)g.units_per_xcd + r
+                            : ((r >> g.xcd_shift) << (g.xcd_shift + 3)) + (x << g.xcd_shift) +
+                                  (r & ((1u << g.xcd_shift) - 1u));
+  if (unit >= (unsigned)g.total_units) return false;
   // the groups of one (tile, segment) are neighbours in launch order: they stream the same
   // upstream-gradient rows at about the same time, through the same L2
-  const int per_tile = g.nseg * g.ngroups;
-  const int64_t tile = unit / per_tile;
+  const unsigned per_tile = (unsigned)(g.nseg * g.ngroups);
+  const unsigned tile = unit / per_tile;
   const int rem = (int)(unit - tile * per_tile);
   const int segi = rem / g.ngroups;
   t.view0 = (rem - segi * g.ngroups) * g.vper;
   t.d_lo = segi * g.seg;
   t.d_hi = min((int)a.D, t.d_lo + g.seg);
-  t.b = (int)(tile / g.tiles_per_image);
-  const int t_in = (int)(tile - (int64_t)t.b * g.tiles_per_image);
+  t.b = (int)(tile / (unsigned)g.tiles_per_image);
+  const int t_in = (int)(tile - (unsigned)t.b * (unsigned)g.tiles_per_image);
   t.p = t.lane / LPP;
   t.cl = t.lane % LPP;
   t.pin = t_in * PPW + t.p;
@@ -740,18 +745,18 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     float r_scl = 0.f;
     float4 r_wts[NV], r_dwt[NV];
     // Issue the loads of this chunk's cost_grad rows now, unconditionally, so that the
-    // reprojection below overlaps their latency.  They are ordinary (cached) loads: the
-    // workgroup of the next view reads the same rows a moment later and should find them
-    // in L2.
+    // reprojection below overlaps their latency.  Streaming loads: cached ones let the
+    // next view's workgroup hit L2 more often (690 -> 660 MB fetched) and save 10 us here,
+    // but leave the caches full of these rows and cost the next forward launch 25 us.
     float cgr[PF][VEC];
 #pragma unroll
     for (int jj = 0; jj < PF; ++jj) {
       const int d = min(d0 + jj, d_hi - 1);
       const S *src_cg = cg_lane + (int64_t)d * OC;
       if (CORR == 0)
-        load_vec<S, VEC, false>(src_cg, cgr[jj]);
+        load_vec<S, VEC, true>(src_cg, cgr[jj]);
       else
-        load_groups<S, VEC, false>(src_cg, cgr[jj], g.sub);
+        load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
     }
     {
       const float depth = d0 + t.cl < d_hi ? (per_voxel_depth ? dv : base + dv) : 1.f;
@@ -836,9 +841,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
             const int dd = min(d0 + PF + j2, d_hi - 1);
             const S *src_cg = cg_lane + (int64_t)dd * OC;
             if (CORR == 0)
-              load_vec<S, VEC, false>(src_cg, cgr[j2]);
+              load_vec<S, VEC, true>(src_cg, cgr[j2]);
             else
-              load_groups<S, VEC, false>(src_cg, cgr[j2], g.sub);
+              load_groups<S, VEC, true>(src_cg, cgr[j2], g.sub);
           }
         }
       }
@@ -1032,11 +1037,11 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   g.nseg = (int)((D + g.seg - 1) / g.seg);
   g.total_units = tiles * g.nseg * g.ngroups;
   g.units_per_xcd = (g.total_units + 7) / 8;
-  // backward: about 32 units per run, whole pixel tiles (their view groups share L2 lines)
-  const int per_tile = g.nseg * g.ngroups;
-  g.xcd_run = vper > 0 ? per_tile * (32 / per_tile > 1 ? 32 / per_tile : 1)
-                       : (int)(g.units_per_xcd > 0 ? g.units_per_xcd : 1);
-  g.grid = (g.total_units + 8 * (int64_t)g.xcd_run - 1) / (8 * (int64_t)g.xcd_run) * (8 * (int64_t)g.xcd_run);
+  // backward: runs of 32 units (the view groups of a tile are neighbours and mostly share
+  // a run, hence an L2)
+  g.xcd_shift = vper > 0 ? 5 : -1;
+  const int64_t round_to = vper > 0 ? 8 * 32 : 8;
+  g.grid = vper > 0 ? (g.total_units + round_to - 1) / round_to * round_to : g.units_per_xcd * 8;
   g.sub = sub;
   return g;
 }
