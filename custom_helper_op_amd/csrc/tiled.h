@@ -47,6 +47,7 @@ struct Geometry {
   int xcd_shift;           // log2 of the units dealt to one XCD at a time; -1: one band per XCD
   int64_t grid;            // workgroups to launch
   int sub;                 // channels per correlation group (1 for squared difference)
+  float src_h_max, src_w_max;  // (float)(srcH - 1), (float)(srcW - 1): acceptance bounds
 };
 
 // ---- vector access ---------------------------------------------------------------------
@@ -302,7 +303,8 @@ struct Hit {
 
 template <int NV>
 __device__ __forceinline__ void reproject(const Cameras<NV> &c, int n, float depth, float half,
-                                          int srcH, int srcW, int C, Hit &r) {
+                                          float src_h_max, float src_w_max, int srcW, int C,
+                                          Hit &r) {
   r.off = -1;
   r.key = 0;
   r.k00 = r.k01 = r.k11 = r.k10 = 0.f;
@@ -314,8 +316,7 @@ __device__ __forceinline__ void reproject(const Cameras<NV> &c, int n, float dep
   float sh = r.h3d / r.z;
   sw = sw - half;
   sh = sh - half;
-  if (sh > 0.f && sw > 0.f && sh < static_cast<float>(srcH - 1) &&
-      sw < static_cast<float>(srcW - 1)) {
+  if (sh > 0.f && sw > 0.f && sh < src_h_max && sw < src_w_max) {
     const int fh = static_cast<int>(sh), fw = static_cast<int>(sw);
     r.dh = sh - static_cast<float>(fh);
     r.dw = sw - static_cast<float>(fw);
@@ -343,7 +344,10 @@ constexpr int forward_lds_words(int lpp) {
 }
 
 template <typename S, int VEC, int LPP, int NV, int CORR>
-__global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geometry g) {
+// At most five waves per SIMD: with six (the two-view instantiation needs only 80 VGPRs)
+// the waves of a CU evict each other's taps from L1 and the kernel is 6 % slower.
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void forward_kernel(
+    const Args<S> a, const Geometry g) {
   constexpr int PPW = 64 / LPP;
   extern __shared__ __align__(16) unsigned char smem[];
   Tile<LPP> t;
@@ -391,7 +395,7 @@ __global__ __launch_bounds__(64) void forward_kernel(const Args<S> a, const Geom
         Hit hit;
         hit.off = -1;
         hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
-        if (n < N && d_ok) reproject<NV>(cam, n, depth, half, srcH, srcW, C, hit);
+        if (n < N && d_ok) reproject<NV>(cam, n, depth, half, g.src_h_max, g.src_w_max, srcW, C, hit);
         cnt += hit.off >= 0;
         if constexpr (LPP > 1) {
           lds_at<int>(smem, q4, kOff + (n * LPP * PPW) * 4) = hit.off;
@@ -558,7 +562,8 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
                              (unsigned)(x - nx) < (unsigned)WN::COLS);
       const unsigned long long m = __ballot(leaving);
       if (leaving) {
-        const int rank = count + __popcll(m & ((1ull << lane) - 1ull));
+        const int rank = count + (int)__builtin_amdgcn_mbcnt_hi(
+            (unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));  // leaving lanes below me
         list[2 * rank] = s;
         list[2 * rank + 1] = y * srcW + x;
       }
@@ -619,14 +624,15 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
         const int lead = __ffsll((long long)firing) - 1;
         firing &= ~(((1ull << LPP) - 1ull) << lead);  // retire this pixel's lanes
         if (lane - cl == lead) {
+          vecf old[4];
 #pragma unroll
-          for (int k0 = 0; k0 < 4; k0 += 2) {
-            vecf o0 = *reinterpret_cast<vecf *>(base + slot[k0] * WN::STRIDE);
-            vecf o1 = *reinterpret_cast<vecf *>(base + slot[k0 + 1] * WN::STRIDE);
+          for (int k = 0; k < 4; ++k)
+            old[k] = *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) o0[i] += v[k0][i], o1[i] += v[k0 + 1][i];
-            *reinterpret_cast<vecf *>(base + slot[k0] * WN::STRIDE) = o0;
-            *reinterpret_cast<vecf *>(base + slot[k0 + 1] * WN::STRIDE) = o1;
+          for (int k = 0; k < 4; ++k) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) old[k][i] += v[k][i];
+            *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE) = old[k];
           }
         }
         if (firing) wave_sync();
@@ -699,11 +705,12 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
     const int64_t vo = ((int64_t)t.b * N + (t.view0 + n < N ? t.view0 + n : 0)) * view_elems;
-    view[n] = a.src + vo + t.cl * VEC;
+    view[n] = a.src + vo;  // uniform: taps are addressed as base + 32-bit lane offset
     gview[n] = src_grad_img + vo;
     oy[n] = ox[n] = WN::kNone;
   }
   const int row_step = srcW * C;
+  const unsigned lane_ch = (unsigned)(t.cl * VEC);
 
   float tap[NV][4][VEC], sg[NV][4][VEC];
   int cur[NV];     // tap offset of the open run, -1: none
@@ -773,7 +780,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
         float4 dw4 = make_float4(0.f, 0.f, 0.f, 0.f);
         if (t.view0 + n < N && cnt > 0) {
-          reproject<NV>(cam, n, depth, half, srcH, srcW, C, hit);
+          reproject<NV>(cam, n, depth, half, g.src_h_max, g.src_w_max, srcW, C, hit);
           if (hit.off >= 0) {
             // d(sample)/d(depth) = sum over taps of dwt * tap, from
             //   d/d(src_h) = t1*dw + (t10 - t00),  d/d(src_w) = t1*dh + (t01 - t00),
@@ -830,6 +837,25 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       }
     }
     if constexpr (LPP > 1) wave_sync();
+    int rb_off[2][NV];
+    float4 rb_wt[2][NV], rb_dwt[2][NV];
+    float rb_scl[2];
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      if constexpr (LPP > 1) {
+        rb_off[0][n] = lds_at<int>(smem, p4, kOff + (n * LPP * PPW) * 4);
+        rb_wt[0][n] = lds_at<float4>(smem, p4 * 4u, kWts + (n * LPP * PPW) * 16);
+        rb_dwt[0][n] = lds_at<float4>(smem, p4 * 4u, kDwt + (n * LPP * PPW) * 16);
+      } else {
+        rb_off[0][n] = r_off[n];
+        rb_wt[0][n] = r_wts[n];
+        rb_dwt[0][n] = r_dwt[n];
+      }
+    }
+    if constexpr (LPP > 1)
+      rb_scl[0] = lds_at<float>(smem, p4, kScl);
+    else
+      rb_scl[0] = r_scl;
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
@@ -847,27 +873,23 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           }
         }
       }
-      // this depth's records (LDS broadcasts); the other waves of the SIMD cover the latency
-      int rec_off[NV];
-      float4 rec_wt[NV], rec_dwt[NV];
-      float scl;
+      // The records of the NEXT depth are requested now, so that their LDS latency overlaps
+      // this depth's arithmetic (jj is unrolled: the buffer index is a compile-time constant).
+      const int cb = jj & 1, nb = cb ^ 1;
       if constexpr (LPP > 1) {
+        if (jj + 1 < LPP) {
 #pragma unroll
-        for (int n = 0; n < NV; ++n) {
-          rec_off[n] = lds_at<int>(smem, p4, kOff + ((n * LPP + jj) * PPW) * 4);
-          rec_wt[n] = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj) * PPW) * 16);
-          rec_dwt[n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj) * PPW) * 16);
+          for (int n = 0; n < NV; ++n) {
+            rb_off[nb][n] = lds_at<int>(smem, p4, kOff + ((n * LPP + jj + 1) * PPW) * 4);
+            rb_wt[nb][n] = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj + 1) * PPW) * 16);
+            rb_dwt[nb][n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj + 1) * PPW) * 16);
+          }
+          rb_scl[nb] = lds_at<float>(smem, p4, kScl + ((jj + 1) * PPW) * 4);
         }
-        scl = lds_at<float>(smem, p4, kScl + (jj * PPW) * 4);
-      } else {
-#pragma unroll
-        for (int n = 0; n < NV; ++n) {
-          rec_off[n] = r_off[n];
-          rec_wt[n] = r_wts[n];
-          rec_dwt[n] = r_dwt[n];
-        }
-        scl = r_scl;
       }
+      const int *rec_off = rb_off[cb];
+      const float4 *rec_wt = rb_wt[cb], *rec_dwt = rb_dwt[cb];
+      const float scl = rb_scl[cb];
       float dvox = 0.f;  // this lane's share of d(loss)/d(depth of this voxel)
       if (scl != 0.f) {
         float cg[VEC];
@@ -895,11 +917,15 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
             if (off != cur[n]) {
               // the run on the previous cell ends.  Start fetching the new cell's taps
               // first, then hand the old cell's image to the window while they arrive.
-              const S *q = view[n] + off;
-              load_vec<S, VEC, false>(q, tap[n][0]);
-              load_vec<S, VEC, false>(q + C, tap[n][1]);
-              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
-              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
+              // byte offsets in 32 bits: the loads take the view's base from scalar registers
+              const unsigned e0 = ((unsigned)off + lane_ch) * (unsigned)sizeof(S);
+              const unsigned e1 = e0 + (unsigned)row_step * (unsigned)sizeof(S);
+              const char *vb = reinterpret_cast<const char *>(view[n]);
+              const unsigned cb = (unsigned)C * (unsigned)sizeof(S);
+              load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + e0), tap[n][0]);
+              load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + (e0 + cb)), tap[n][1]);
+              load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + (e1 + cb)), tap[n][2]);
+              load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + e1), tap[n][3]);
               if (cur[n] >= 0)
                 window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
                                      s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
@@ -1043,6 +1069,7 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   const int64_t round_to = vper > 0 ? 8 * 32 : 8;
   g.grid = vper > 0 ? (g.total_units + round_to - 1) / round_to * round_to : g.units_per_xcd * 8;
   g.sub = sub;
+  g.src_h_max = g.src_w_max = 0.f;  // set by the launcher from the source image size
   return g;
 }
 
