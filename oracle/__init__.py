@@ -104,6 +104,45 @@ def cost_volume_bwd(ref, src, base_plane, offsets, Rs, Ts, cost_grad, mask, redu
     return ref_grad, src_grad, bp_grad
 
 
+def cost_aggregate_fwd(ref, src, base_plane, offsets, Rs, Ts, reduce="MEAN", half_centor=True,
+                       threads=1):
+    """cost [B,H,W,D] and mask [B,H,W,D] (MEAN: valid-view count, MIN: winning view or -1)."""
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, base_plane, offsets, Rs, Ts = (_c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts))
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = offsets.shape[1]
+    cost = np.empty((B, H, W, D), dt)
+    mask = np.empty((B, H, W, D), np.int32)
+    fn = getattr(lib(), "chop_oracle_cost_aggregate_fwd_" + sfx)
+    rc = fn(_REDUCE[reduce], int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref),
+            _p(src), _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
+    _check(rc, "cost_aggregate_fwd")
+    return cost, mask
+
+
+def cost_aggregate_bwd(ref, src, base_plane, offsets, Rs, Ts, cost_grad, mask, reduce="MEAN",
+                       half_centor=True, threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, base_plane, offsets, Rs, Ts, cost_grad = (
+        _c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts, cost_grad))
+    mask = _c(mask, np.int32)
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = offsets.shape[1]
+    ref_grad = np.empty_like(ref)
+    src_grad = np.empty_like(src)
+    bp_grad = np.empty_like(base_plane)
+    fn = getattr(lib(), "chop_oracle_cost_aggregate_bwd_" + sfx)
+    rc = fn(_REDUCE[reduce], int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref),
+            _p(src), _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost_grad), _p(mask),
+            _p(ref_grad), _p(src_grad), _p(bp_grad), int(threads))
+    _check(rc, "cost_aggregate_bwd")
+    return ref_grad, src_grad, bp_grad
+
+
 def cost_volume_v2_fwd(ref, src, depth_grid, Rs, Ts, reduce="MEAN", groups=1, half_centor=True,
                        threads=1):
     dt = ref.dtype

@@ -19,12 +19,23 @@
  *       :349-479 CostMeanVolumeGradV2Kernel  -> chop_oracle_cost_volume_v2_bwd_* (reduce 0)
  *       :481-601 CostMinVolumeGradV2Kernel   -> chop_oracle_cost_volume_v2_bwd_* (reduce 1)
  *
+ *   custom_helper_op/cc/kernels/cost_aggregate_kernels_gpu.cu.cc
+ *       :33-126  CostMeanAggregateKernel     -> chop_oracle_cost_aggregate_fwd_* (reduce 0)
+ *       :128-229 CostMinAggregateKernel      -> chop_oracle_cost_aggregate_fwd_* (reduce 1)
+ *       :338-452 CostMeanAggregateGradKernel -> chop_oracle_cost_aggregate_bwd_* (reduce 0)
+ *       :454-563 CostMinAggregateGradKernel  -> chop_oracle_cost_aggregate_bwd_* (reduce 1)
+ *
  * Parity status of each function (what pins it is in tests/test_oracle_*.py):
  *   forward MEAN/MIN (V1), MEAN/MAX (V2): pinned by an independent float64 composite that
  *     restates the reference tests' own oracle, by closed-form camera cases, by a
  *     brute-force Python loop on tiny inputs, and by invariants.
  *   backward, all four: pinned by central finite differences of the forward in float64
  *     with the reference tests' loss and tolerance, and by conservation identities.
+ *   aggregate forward MEAN: pinned against the pinned cost-volume forward (it is its mean
+ *     over channels) and by the composite; MIN: by the composite and brute force.
+ *   aggregate backward: MEAN pinned against the pinned cost-volume backward fed the
+ *     upstream gradient broadcast over channels and divided by C; both reduces by finite
+ *     differences in float64.
  *   sample_coords: pinned by the float64 composite's coordinates.
  *   NOT pinned: the rounding of a CUDA build of the reference (nvcc contracts a*b+c into
  *     fused multiply-adds and the reference is built with ftz=true).  No such build or
