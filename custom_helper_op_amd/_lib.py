@@ -23,6 +23,8 @@ SIGNATURES = {
 for _t in ("f32", "f64"):
     SIGNATURES["chop_cost_volume_fwd_" + _t] = [_vp, _int, _int] + _DIMS + [_vp] * 8
     SIGNATURES["chop_cost_volume_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_vp] * 11
+    SIGNATURES["chop_cost_aggregate_fwd_" + _t] = [_vp, _int, _int] + _DIMS + [_vp] * 8
+    SIGNATURES["chop_cost_aggregate_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_vp] * 11
     SIGNATURES["chop_cost_volume_v2_fwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 7
     SIGNATURES["chop_cost_volume_v2_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 10
     SIGNATURES["chop_cost_volume_sample_coords_" + _t] = [_vp, _int] + [_i64] * 7 + [_vp] * 10

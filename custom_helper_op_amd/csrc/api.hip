@@ -232,6 +232,47 @@ int chop_cost_volume_bwd_f64(void *stream, int reduce, int half_centor, int64_t 
                           src_grad, base_plane_grad, false, nullptr, 0);
 }
 
+int chop_cost_aggregate_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const float *ref, const float *src,
+                                const float *base_plane, const float *offsets, const float *Rs,
+                                const float *Ts, float *cost, int32_t *mask) {
+  return forward<float>(stream, reduce, half_centor, DIMS, 1, SUM_SQUARED_DIFFERENCE, ref, src,
+                        base_plane, offsets, nullptr, Rs, Ts, cost, mask, false);
+}
+
+int chop_cost_aggregate_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const double *ref, const double *src,
+                                const double *base_plane, const double *offsets,
+                                const double *Rs, const double *Ts, double *cost, int32_t *mask) {
+  return forward<double>(stream, reduce, half_centor, DIMS, 1, SUM_SQUARED_DIFFERENCE, ref, src,
+                         base_plane, offsets, nullptr, Rs, Ts, cost, mask, false);
+}
+
+int chop_cost_aggregate_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const float *ref, const float *src,
+                                const float *base_plane, const float *offsets, const float *Rs,
+                                const float *Ts, const float *cost_grad, const int32_t *mask,
+                                float *ref_grad, float *src_grad, float *base_plane_grad) {
+  return backward<float>(stream, reduce, half_centor, DIMS, 1, SUM_SQUARED_DIFFERENCE, ref, src,
+                         base_plane, offsets, nullptr, Rs, Ts, cost_grad, mask, ref_grad, src_grad,
+                         base_plane_grad, false, nullptr, 0);
+}
+
+int chop_cost_aggregate_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const double *ref, const double *src,
+                                const double *base_plane, const double *offsets,
+                                const double *Rs, const double *Ts, const double *cost_grad,
+                                const int32_t *mask, double *ref_grad, double *src_grad,
+                                double *base_plane_grad) {
+  return backward<double>(stream, reduce, half_centor, DIMS, 1, SUM_SQUARED_DIFFERENCE, ref, src,
+                          base_plane, offsets, nullptr, Rs, Ts, cost_grad, mask, ref_grad,
+                          src_grad, base_plane_grad, false, nullptr, 0);
+}
+
 int chop_cost_volume_v2_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
                                 int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
                                 int64_t srcW, int groups, const float *ref, const float *src,

@@ -98,6 +98,53 @@ __global__ __launch_bounds__(kBlock) void general_forward_kernel(const Args<S> a
   }
 }
 
+// CostAggregate forward: one thread per voxel, channels and views serial, in the order of
+// cost_aggregate_kernels_gpu.cu.cc:75-124 (MEAN) and :173-228 (MIN).
+template <typename S, int REDUCE>
+__global__ __launch_bounds__(kBlock) void general_aggregate_forward_kernel(const Args<S> a) {
+  using R = typename Storage<S>::Real;
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int64_t total = a.voxels();
+  const int64_t row_step = (int64_t)srcW * C;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * kBlock) {
+    const Voxel<R> v = locate(a, i);
+    const S *ref_px = a.ref + v.pix * C;
+    R acc = REDUCE == 0 ? R(0) : Limits<R>::max();
+    int used = REDUCE == 0 ? 0 : -1;
+    for (int n = 0; n < N; ++n) {
+      Sample<R> s;
+      const int64_t cam = (int64_t)v.b * N + n;
+      project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+      if (s.state != 2) continue;
+      const S *t00 = a.src + (int64_t)C * (s.fw + (int64_t)srcW * (s.fh + (int64_t)srcH * cam));
+      const S *t01 = t00 + C, *t11 = t01 + row_step, *t10 = t00 + row_step;
+      R cur = REDUCE == 0 ? acc : R(0);
+      for (int c = 0; c < C; ++c) {
+        const R smp = s.k00 * Storage<S>::load(t00 + c) + s.k01 * Storage<S>::load(t01 + c) +
+                      s.k11 * Storage<S>::load(t11 + c) + s.k10 * Storage<S>::load(t10 + c);
+        const R diff = smp - Storage<S>::load(ref_px + c);
+        cur += diff * diff;
+      }
+      if (REDUCE == 0) {
+        acc = cur;
+        ++used;
+      } else if (acc > cur) {
+        acc = cur;
+        used = n;
+      }
+    }
+    a.mask[i] = used;
+    R out = R(0);
+    if (REDUCE == 0) {
+      if (used > 0) out = acc / static_cast<R>((int64_t)used * C);
+    } else if (used >= 0) {
+      out = acc / static_cast<R>(C);
+    }
+    Storage<S>::store(a.cost + i, out);
+  }
+}
+
 template <typename S, int CORR, int REDUCE>
 __global__ __launch_bounds__(kBlock) void general_backward_kernel(const Args<S> a) {
   using R = typename Storage<S>::Real;
@@ -105,22 +152,26 @@ __global__ __launch_bounds__(kBlock) void general_backward_kernel(const Args<S> 
   Acc *ref_grad = Is16<S>::value ? (Acc *)a.ref_grad_acc : (Acc *)a.ref_grad;
   Acc *src_grad = Is16<S>::value ? (Acc *)a.src_grad_acc : (Acc *)a.src_grad;
   const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  const int OC = CORR ? a.groups : C;
-  const int sub = CORR ? C / a.groups : 1;
+  // CORR == 2 (CostAggregate, cost_aggregate_kernels_gpu.cu.cc:338-563): one upstream
+  // gradient and one mask entry per voxel, shared by all channels
+  const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
+  const int sub = CORR == 1 ? C / a.groups : 1;
   const int64_t total = a.voxels() * C;
   const int64_t row_step = (int64_t)srcW * C;
   for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total;
        e += (int64_t)gridDim.x * kBlock) {
     const int64_t i = e / C;
     const int c = (int)(e - i * C);
-    const int oc = CORR ? c / sub : c;
+    const int oc = CORR == 1 ? c / sub : CORR == 2 ? 0 : c;
     const int32_t *mrow = a.mask_in + (REDUCE == 0 ? i : i * OC);
     const int32_t m0 = mrow[0];
     if (REDUCE == 0 ? (m0 <= 0) : (m0 < 0)) continue;  // depth gradient stays at its zero fill
     const int32_t winner = REDUCE == 0 ? 0 : mrow[oc];
     const Voxel<R> v = locate(a, i);
     const R ref_c = Storage<S>::load(a.ref + v.pix * C + c);
-    const R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
+    R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
+    if (CORR == 2)  // :388 cost_grad / (T)(mask * channels), :502 cost_grad / (T)channels
+      cg = REDUCE == 0 ? cg / static_cast<R>((int64_t)m0 * C) : cg / static_cast<R>(C);
     R depth_grad = R(0);
     for (int n = 0; n < N; ++n) {
       Sample<R> s;
@@ -137,6 +188,10 @@ __global__ __launch_bounds__(kBlock) void general_backward_kernel(const Args<S> 
       if (CORR == 0) {
         const R diff = smp - ref_c;
         g = REDUCE == 0 ? R(2) * diff * cg / static_cast<R>(m0) : R(2) * diff * cg;
+        atomic_add(ref_grad + v.pix * C + c, (Acc)(-g));
+      } else if (CORR == 2) {
+        const R diff = smp - ref_c;
+        g = R(2) * diff * cg;
         atomic_add(ref_grad + v.pix * C + c, (Acc)(-g));
       } else {
         g = REDUCE == 0 ? cg / static_cast<R>(m0) : cg;
@@ -234,7 +289,12 @@ hipError_t launch_general_forward(const Args<S> &a, hipStream_t stream) {
   const int64_t total = a.voxels() * a.out_channels();
   if (total == 0) return hipSuccess;
   const int grid = grid_for(total, kBlock);
-  if (a.corr == SQUARED_DIFFERENCE) {
+  if (a.corr == SUM_SQUARED_DIFFERENCE) {
+    if (a.reduce == 0)
+      general_aggregate_forward_kernel<S, 0><<<grid, kBlock, 0, stream>>>(a);
+    else
+      general_aggregate_forward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  } else if (a.corr == SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
       general_forward_kernel<S, 0, 0><<<grid, kBlock, 0, stream>>>(a);
     else
@@ -266,7 +326,12 @@ hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream) {
   const int64_t total = a.voxels() * a.C;
   if (total > 0) {
     const int grid = grid_for(total, kBlock);
-    if (a.corr == SQUARED_DIFFERENCE) {
+    if (a.corr == SUM_SQUARED_DIFFERENCE) {
+      if (a.reduce == 0)
+        general_backward_kernel<S, 2, 0><<<grid, kBlock, 0, stream>>>(a);
+      else
+        general_backward_kernel<S, 2, 1><<<grid, kBlock, 0, stream>>>(a);
+    } else if (a.corr == SQUARED_DIFFERENCE) {
       if (a.reduce == 0)
         general_backward_kernel<S, 0, 0><<<grid, kBlock, 0, stream>>>(a);
       else

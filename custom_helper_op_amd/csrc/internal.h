@@ -9,7 +9,11 @@
 
 namespace chop {
 
-enum Corr { SQUARED_DIFFERENCE = 0, GROUP_CORRELATION = 1 };
+// What the per-view term is and what a cost row holds:
+//   SQUARED_DIFFERENCE      (sample - ref)^2 per channel              row = C values
+//   GROUP_CORRELATION       sum over a channel group of sample * ref  row = groups values
+//   SUM_SQUARED_DIFFERENCE  (sample - ref)^2 summed over the channels row = 1 value (CostAggregate)
+enum Corr { SQUARED_DIFFERENCE = 0, GROUP_CORRELATION = 1, SUM_SQUARED_DIFFERENCE = 2 };
 
 // One call's arguments after validation.  S = storage type of the feature tensors,
 // R = Storage<S>::Real = type of depth inputs, camera matrices, depth gradients.
@@ -38,7 +42,9 @@ struct Args {
 
   __host__ __device__ int64_t pixels() const { return B * H * W; }
   __host__ __device__ int64_t voxels() const { return B * H * W * D; }
-  __host__ __device__ int out_channels() const { return corr == GROUP_CORRELATION ? groups : (int)C; }
+  __host__ __device__ int out_channels() const {
+    return corr == GROUP_CORRELATION ? groups : corr == SUM_SQUARED_DIFFERENCE ? 1 : (int)C;
+  }
 };
 
 // General kernels: any shape, any channel count, both reduces, all storage types.

@@ -1,8 +1,8 @@
 """Host-side mirror of the reference's Python operator interface for the cost volume.
 
 Same names, argument order, defaults and outputs as
-custom_helper_op/python/ops/custom_helper_ops.py:32-96 (``cost_volume``,
-``cost_volume_v2`` and the gradients registered for them), with torch tensors standing in
+custom_helper_op/python/ops/custom_helper_ops.py:32-96 and :133-163 (``cost_volume``,
+``cost_volume_v2``, ``cost_aggregate`` and the gradients registered for them), with torch tensors standing in
 for TensorFlow tensors: torch supplies device memory and the current HIP stream, the
 arithmetic is done by ``libchop_costvol.so`` through its C ABI.  The shape checks are the
 ones ``CostVolumeOp::Compute`` performs (custom_helper_op/cc/kernels/
@@ -228,6 +228,63 @@ def cost_volume_grad_v2(ref_image, src_images, depth_grid, rs, ts, cost_grad, co
     return ref_grad, src_grad, dg_grad
 
 
+def cost_aggregate_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
+                       half_centor=True):
+    """The ``CostAggregate`` op without autograd: ``(cost [B,H,W,D], cost_mask int32 [B,H,W,D])``
+    (shapes: custom_helper_op/cc/ops/custom_helper_ops.cc:46-58; checks:
+    cost_aggregate_kernels.cc:85-106).  float32 and float64 only, as registered."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, dt, dev, "base_plane")
+    offsets = _prep(offsets, dt, dev, "offsets")
+    Rs, Ts = _prep(Rs, dt, dev, "Rs"), _prep(Ts, dt, dev, "Ts")
+    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, Rs, Ts)
+    cost = torch.empty((B, H, W, D), dtype=dt, device=dev)
+    mask = torch.empty((B, H, W, D), dtype=torch.int32, device=dev)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    fn = lib.chop_cost_aggregate_fwd_f32 if dt == torch.float32 else lib.chop_cost_aggregate_fwd_f64
+    rc = fn(_stream(cost), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
+            _ptr(base_plane), _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(cost), _ptr(mask))
+    _lib.check(rc)
+    return cost, mask
+
+
+def cost_aggregate_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_grad, cost_mask,
+                        reduce_method="MEAN", half_centor=True):
+    """The ``CostAggregateGrad`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``
+    (checks: cost_aggregate_kernels.cc:196-226)."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, dt, dev, "base_plane")
+    offsets = _prep(offsets, dt, dev, "offsets")
+    rs, ts = _prep(rs, dt, dev, "Rs"), _prep(ts, dt, dev, "Ts")
+    cost_grad = _prep(cost_grad, dt, dev, "cost_grad")
+    cost_mask = _prep(cost_mask, torch.int32, dev, "cost_mask")
+    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, rs, ts)
+    _require(tuple(cost_grad.shape) == (B, H, W, D),
+             "cost_grad must have rank 4, and must compate to ref_image")
+    _require(tuple(cost_mask.shape) == (B, H, W, D),
+             "cost_mask must have rank 4, and must compate to ref_image")
+    ref_grad = torch.empty_like(ref_image)
+    src_grad = torch.empty_like(src_images)
+    bp_grad = torch.empty_like(base_plane)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    fn = lib.chop_cost_aggregate_bwd_f32 if dt == torch.float32 else lib.chop_cost_aggregate_bwd_f64
+    rc = fn(_stream(ref_grad), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
+            _ptr(base_plane), _ptr(offsets), _ptr(rs), _ptr(ts), _ptr(cost_grad), _ptr(cost_mask),
+            _ptr(ref_grad), _ptr(src_grad), _ptr(bp_grad))
+    _lib.check(rc)
+    return ref_grad, src_grad, bp_grad
+
+
 class _CostVolume(torch.autograd.Function):
     """Forward = CostVolume, backward = the gradient registered for it
     (custom_helper_ops.py:41-61): the Grad op is fed the forward's cost_mask, the incoming
@@ -270,6 +327,26 @@ class _CostVolumeV2(torch.autograd.Function):
         return rg, sg, dg, None, None, None, None, None
 
 
+class _CostAggregate(torch.autograd.Function):
+    """CostAggregate with its registered gradient (custom_helper_ops.py:141-161)."""
+
+    @staticmethod
+    def forward(ctx, ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method, half_centor):
+        cost, mask = cost_aggregate_raw(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                        reduce_method, half_centor)
+        ctx.save_for_backward(ref_image, src_images, base_plane, offsets, Rs, Ts, mask)
+        ctx.attrs = (reduce_method, half_centor)
+        ctx.mark_non_differentiable(mask)
+        return cost, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        ref_image, src_images, base_plane, offsets, Rs, Ts, mask = ctx.saved_tensors
+        rg, sg, bg = cost_aggregate_grad(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                         grad_out.contiguous(), mask, *ctx.attrs)
+        return rg, sg, bg, None, None, None, None, None
+
+
 def cost_volume(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
                 half_centor=True, name=None):
     """``custom_helper_op.cost_volume``: returns ``(cost, cost_mask)``; differentiable with
@@ -291,6 +368,19 @@ def cost_volume_v2(ref_image, src_images, depth_grid, Rs, Ts, reduce_method="MEA
     Ts = torch.as_tensor(Ts, device=ref_image.device)
     return _CostVolumeV2.apply(ref_image, src_images, depth_grid, Rs, Ts, reduce_method, groups,
                                half_centor)
+
+
+def cost_aggregate(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
+                   half_centor=True, name=None):
+    """``custom_helper_op.cost_aggregate`` (custom_helper_ops.py:133-138): returns
+    ``(cost [B,H,W,D], cost_mask [B,H,W,D])``; differentiable with respect to ref_image,
+    src_images and base_plane."""
+    del name
+    offsets = torch.as_tensor(offsets, device=ref_image.device)
+    Rs = torch.as_tensor(Rs, device=ref_image.device)
+    Ts = torch.as_tensor(Ts, device=ref_image.device)
+    return _CostAggregate.apply(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method,
+                                half_centor)
 
 
 def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):

@@ -119,6 +119,42 @@ int chop_cost_volume_v2_bwd_f64(void *stream, int reduce, int half_centor, int64
                                 const double *cost_grad, const int32_t *mask, double *ref_grad,
                                 double *src_grad, double *depth_grid_grad);
 
+/* ---- CostAggregate forward / backward -----------------------------------------------
+ * The squared differences of all channels summed into one value per voxel.
+ * Replaces functor::CostAggregateFunctor<GPUDevice,T,half_centor>::operator() and
+ * functor::CostAggregateGradFunctor<GPUDevice,T,half_centor>::operator()
+ * (declared custom_helper_op/cc/kernels/cost_aggregate.h:38-133, defined
+ * cost_aggregate_kernels_gpu.cu.cc:290-331 and :586-646, called from
+ * CostAggregateOp::Compute and CostAggregateGradOp::Compute,
+ * cost_aggregate_kernels.cc:120-128 and :247-255).
+ * cost is [B,H,W,D]; mask is int32 [B,H,W,D]: the number of accepted views (MEAN) or the
+ * view with the smallest sum, -1 if none was accepted (MIN).  MEAN divides the sum by
+ * (accepted views * C), MIN by C; a voxel no view accepted gets cost 0.
+ * The backward takes cost_grad [B,H,W,D] and the forward's mask. */
+int chop_cost_aggregate_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const float *ref, const float *src,
+                                const float *base_plane, const float *offsets, const float *Rs,
+                                const float *Ts, float *cost, int32_t *mask);
+int chop_cost_aggregate_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const double *ref, const double *src,
+                                const double *base_plane, const double *offsets,
+                                const double *Rs, const double *Ts, double *cost, int32_t *mask);
+int chop_cost_aggregate_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const float *ref, const float *src,
+                                const float *base_plane, const float *offsets, const float *Rs,
+                                const float *Ts, const float *cost_grad, const int32_t *mask,
+                                float *ref_grad, float *src_grad, float *base_plane_grad);
+int chop_cost_aggregate_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, const double *ref, const double *src,
+                                const double *base_plane, const double *offsets,
+                                const double *Rs, const double *Ts, const double *cost_grad,
+                                const int32_t *mask, double *ref_grad, double *src_grad,
+                                double *base_plane_grad);
+
 /* ---- 16-bit storage extension --------------------------------------------------------
  * No counterpart in the reference, whose ops register float32 and float64 only
  * (custom_helper_ops.cc:197,234).  ref, src, cost, cost_grad, ref_grad and src_grad
