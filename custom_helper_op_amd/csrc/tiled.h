@@ -164,10 +164,21 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// Sum over each group of WIDTH consecutive lanes (WIDTH a power of two <= 16), left in every
+// lane of the group.  Cross-lane moves in registers: quad permutes, then the half-row and
+// row mirrors (a mirror pairs lane i with lane WIDTH-1-i; the quad steps finish the sum).
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+  return v + __int_as_float(moved);
+}
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int m = WIDTH / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, WIDTH);
+  static_assert(WIDTH == 1 || WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16, "group width");
+  if constexpr (WIDTH >= 16) v = dpp_add<0x140>(v);  // row_mirror
+  if constexpr (WIDTH >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+  if constexpr (WIDTH >= 4) v = dpp_add<0x4E>(v);    // quad_perm 2,3,0,1
+  if constexpr (WIDTH >= 2) v = dpp_add<0xB1>(v);    // quad_perm 1,0,3,2
   return v;
 }
 
@@ -378,7 +389,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
 #pragma unroll
   for (int n = 0; n < NV; ++n) cur[n] = -1;
 
-  const int OC = CORR ? a.groups : C;
+  // CORR: 0 squared difference per channel, 1 group correlation, 2 squared difference
+  // summed over all channels (one value per voxel)
+  const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
   const int gv = VEC / g.sub;  // output values per lane
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
@@ -409,6 +422,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
     }
     if constexpr (LPP > 1) wave_sync();
+    float agg_out = 0.f;
     // ---- phase 2: channel arithmetic by lane (p, channel slice) ---------------------------
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
@@ -440,7 +454,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           }
 #pragma unroll
           for (int c = 0; c < VEC; ++c) {
-            if (CORR == 0) {
+            if (CORR != 1) {
               // sample - ref as one chain of fused multiply-adds
               float diff = __builtin_fmaf(wt.x, tap[n][0][c], -ref[c]);
               diff = __builtin_fmaf(wt.y, tap[n][1][c], diff);
@@ -458,6 +472,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           ++k;
         }
       }
+      if constexpr (CORR == 2) {
+        // one value per voxel: the pixel's lanes add up their channels; the lane whose
+        // slice index equals the depth's place in the chunk keeps the result, so that the
+        // chunk is stored as LPP consecutive floats per pixel
+        float tot = group_sum<LPP>((acc[0] + acc[1]) + (acc[2] + acc[3]));
+        tot = k > 0 ? tot / static_cast<float>(k * C) : 0.f;
+        if constexpr (LPP > 1) {
+          if (t.cl == jj) agg_out = tot;
+        } else {
+          if (t.pix_ok) __builtin_nontemporal_store(tot, reinterpret_cast<float *>(a.cost) + t.pix * D + d);
+        }
+        continue;
+      }
       if (k > 1) {
         const float inv = __builtin_amdgcn_rcpf(static_cast<float>(k));
 #pragma unroll
@@ -473,6 +500,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
         }
       }
+    }
+    if constexpr (CORR == 2 && LPP > 1) {
+      if (t.pix_ok && d0 + t.cl < d_hi)
+        __builtin_nontemporal_store(agg_out, reinterpret_cast<float *>(a.cost) + t.pix * D + d0 + t.cl);
     }
     if constexpr (LPP > 1) wave_sync();
   }
@@ -730,22 +761,26 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   float dacc = 0.f;  // base-plane gradient partial of this lane
   wave_sync();
 
-  const int OC = CORR ? a.groups : C;
+  // CORR: 0 squared difference per channel, 1 group correlation, 2 squared difference
+  // summed over all channels (one upstream gradient per voxel)
+  const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   constexpr int PF = LPP < 8 ? LPP : 8;  // upstream-gradient rows fetched ahead
-  const S *cg_lane = a.cost_grad + t.pix * D * OC + t.cl * (CORR ? gv : VEC);
+  const S *cg_lane = a.cost_grad + t.pix * D * OC + (CORR == 2 ? 0 : t.cl * (CORR ? gv : VEC));
   const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
   const int32_t *cnt_src = a.mask_in + t.pix * D;
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
     // Depth hypothesis and valid-view count of lane (p, j)'s voxel: requested before the
     // chunk's upstream-gradient rows, because loads return in order and the reprojection
     // should wait for these two words only.
-    float dv = 1.f;
+    float dv = 1.f, cg_vox = 0.f;
     int cnt = 0;
     if (d0 + t.cl < d_hi) {
       dv = dv_src[d0 + t.cl];
       if (t.pix_ok) cnt = cnt_src[d0 + t.cl];
+      if constexpr (CORR == 2)  // the voxel's one upstream gradient rides with its record
+        cg_vox = reinterpret_cast<const float *>(cg_lane)[d0 + t.cl];
     }
     int r_off[NV];
     int2 r_cell[NV];
@@ -755,23 +790,30 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     // reprojection below overlaps their latency.  Streaming loads: cached ones let the
     // next view's workgroup hit L2 more often (690 -> 660 MB fetched) and save 10 us here,
     // but leave the caches full of these rows and cost the next forward launch 25 us.
-    float cgr[PF][VEC];
+    float cgr[CORR == 2 ? 1 : PF][VEC];
+    if constexpr (CORR != 2) {
 #pragma unroll
-    for (int jj = 0; jj < PF; ++jj) {
-      const int d = min(d0 + jj, d_hi - 1);
-      const S *src_cg = cg_lane + (int64_t)d * OC;
-      if (CORR == 0)
-        load_vec<S, VEC, true>(src_cg, cgr[jj]);
-      else
-        load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
+      for (int jj = 0; jj < PF; ++jj) {
+        const int d = min(d0 + jj, d_hi - 1);
+        const S *src_cg = cg_lane + (int64_t)d * OC;
+        if (CORR == 0)
+          load_vec<S, VEC, true>(src_cg, cgr[jj]);
+        else
+          load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
+      }
     }
     {
       const float depth = d0 + t.cl < d_hi ? (per_voxel_depth ? dv : base + dv) : 1.f;
       // factor the reduce applies to the upstream gradient: squared difference 2/k,
-      // correlation 1/k; zero marks a voxel no view saw
-      const float scl = cnt > 0 ? (CORR == 0 ? 2.f : 1.f) *
-                                      __builtin_amdgcn_rcpf(static_cast<float>(cnt))
-                                : 0.f;
+      // correlation 1/k, summed squared difference 2*cost_grad/(k*C) (the whole per-voxel
+      // factor); zero marks a voxel that contributes nothing
+      float scl = 0.f;
+      if (cnt > 0) {
+        if constexpr (CORR == 2)
+          scl = 2.f * (cg_vox / static_cast<float>(cnt * C));
+        else
+          scl = (CORR == 0 ? 2.f : 1.f) * __builtin_amdgcn_rcpf(static_cast<float>(cnt));
+      }
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
         Hit hit;
@@ -860,7 +902,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
       if (d >= d_hi) break;
-      if constexpr (LPP > PF) {
+      if constexpr (LPP > PF && CORR != 2) {
         if (jj == PF) {  // second half of a 16-deep chunk
 #pragma unroll
           for (int j2 = 0; j2 < PF; ++j2) {
@@ -894,8 +936,11 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       if (scl != 0.f) {
         float cg[VEC];
         {
-          const float *raw = cgr[jj % PF];
-          if (CORR == 0 || g.sub == 1) {
+          const float *raw = cgr[CORR == 2 ? 0 : jj % PF];
+          if constexpr (CORR == 2) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) cg[c] = scl;
+          } else if (CORR == 0 || g.sub == 1) {
 #pragma unroll
             for (int c = 0; c < VEC; ++c) cg[c] = raw[c] * scl;
           } else if (g.sub == 2) {
@@ -939,7 +984,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
               float gsrc;  // d(loss)/d(sample of this channel)
-              if (CORR == 0) {
+              if (CORR != 1) {
                 float diff = __builtin_fmaf(wt.x, tap[n][0][c], -ref[c]);
                 diff = __builtin_fmaf(wt.y, tap[n][1][c], diff);
                 diff = __builtin_fmaf(wt.z, tap[n][2][c], diff);

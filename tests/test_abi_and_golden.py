@@ -28,7 +28,7 @@ def declared_functions():
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = declared_functions()
-    assert len(names) == 19
+    assert len(names) == 23
     for n in names:
         assert hasattr(lib, n), n
     assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
@@ -40,7 +40,7 @@ def test_oracle_exports():
     lib = oracle.lib()
     for sfx in ("f32", "f64"):
         for stem in ("cost_volume_fwd", "cost_volume_bwd", "cost_volume_v2_fwd", "cost_volume_v2_bwd",
-                     "sample_coords"):
+                     "cost_aggregate_fwd", "cost_aggregate_bwd", "sample_coords"):
             assert hasattr(lib, "chop_oracle_%s_%s" % (stem, sfx))
 
 
@@ -58,6 +58,12 @@ def test_validation_runs_before_any_device_call():
     assert _fwd_f32(lib, 0, (1, -4, 5, 8, 3, 2, 4, 5), fake) == 2
     assert _fwd_f32(lib, 0, (1, 2 ** 40, 5, 8, 3, 2, 4, 5), fake) == 2
     assert _fwd_f32(lib, 0, good, null) == 1 and b"null pointer: ref" in lib.chop_last_error_string()
+    # CostAggregate goes through the same validation
+    assert lib.chop_cost_aggregate_fwd_f32(None, 7, 1, *good, *fake) == 3
+    assert lib.chop_cost_aggregate_fwd_f64(None, 0, 1, *good, *null) == 1
+    assert lib.chop_cost_aggregate_bwd_f32(None, 0, 1, *good, *([None] * 11)) == 1
+    assert lib.chop_cost_aggregate_bwd_f32(None, 0, 1, 1, 4, 5, 8, 0, 2, 4, 5, *([None] * 8),
+                                           *fake[:3]) in (0, 5)  # D = 0: only zero fills
     # zero-sized work: success without touching anything
     assert _fwd_f32(lib, 0, (1, 0, 5, 8, 3, 2, 0, 5), null) == 0
     assert _fwd_f32(lib, 0, (1, 4, 5, 8, 0, 2, 4, 5), null) == 0

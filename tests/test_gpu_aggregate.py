@@ -34,6 +34,13 @@ def _args(t):
     return tuple(t[k] for k in KEYS)
 
 
+def _expect_family(family, C, reduce, dtype):
+    """The tiled kernels take float32 MEAN with a channel count that is 4 times a power of two."""
+    tiled = family == 0 and reduce == "MEAN" and dtype == np.float32 and C in (4, 8, 16, 32, 64)
+    got = _lib.load().chop_last_kernel_family()
+    assert got == (2 if tiled else 1), (got, family, C, reduce, dtype)
+
+
 @pytest.mark.parametrize("family", FAMILIES)
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
@@ -45,6 +52,7 @@ def test_forward(oracle, family, shape, reduce, dtype):
         t = reference_test_case(case, B, N, H, W, C, D, dtype, seed=case)
         want_cost, want_mask = oracle.cost_aggregate_fwd(*_args(t), reduce)
         cost, mask = chop.cost_aggregate_raw(*_inputs(t), reduce)
+        _expect_family(family, C, reduce, dtype)
         assert cost.shape == (B, H, W, D) and mask.shape == (B, H, W, D)
         if reduce == "MEAN" or _lib.load().chop_last_kernel_family() == 1:
             assert np.array_equal(host(mask), want_mask)
@@ -73,6 +81,7 @@ def test_backward(oracle, family, shape, reduce, dtype):
         cg = rng.standard_normal((B, H, W, D)).astype(dtype)
         want = oracle.cost_aggregate_bwd(*_args(t), cg, mask, reduce)
         got = chop.cost_aggregate_grad(*_inputs(t), dev(cg), dev(mask), reduce)
+        _expect_family(family, C, reduce, dtype)
         tol = 1e-4 if dtype == np.float32 else 1e-10
         for g, w in zip(got, want):
             assert g.shape == w.shape
@@ -128,3 +137,20 @@ def test_errors_and_empty():
     # zero depth hypotheses: a successful no-op
     cost, mask = chop.cost_aggregate_raw(x[0], x[1], x[2], x[3][:, :0], x[4], x[5])
     assert cost.shape == (1, 6, 8, 0) and mask.shape == (1, 6, 8, 0)
+
+
+def test_mvsnet_stage_full_size(oracle):
+    """The benchmark workload's tensors through CostAggregate (forward and backward)."""
+    wl = make_workload(2, with_cost_grad=False)
+    t = wl.tensors
+    want_cost, want_mask = oracle.cost_aggregate_fwd(*_args(t), "MEAN", threads=8)
+    cost, mask = chop.cost_aggregate_raw(*_inputs(t), "MEAN")
+    assert _lib.load().chop_last_kernel_family() == 2
+    assert np.array_equal(host(mask), want_mask)
+    assert_forward_close(host(cost), want_cost)
+    cg = np.random.default_rng(9).standard_normal(want_cost.shape).astype(np.float32)
+    want = oracle.cost_aggregate_bwd(*_args(t), cg, want_mask, "MEAN", threads=8)
+    got = chop.cost_aggregate_grad(*_inputs(t), dev(cg), mask, "MEAN")
+    assert _lib.load().chop_last_kernel_family() == 2
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
