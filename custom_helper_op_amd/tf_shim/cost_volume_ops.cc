@@ -9,7 +9,8 @@
 //       -L<repo>/custom_helper_op_amd -lchop_costvol -o _custom_helper_ops.so
 //
 // Drop-in contract (what must not change, with the reference lines that fix it):
-//   op names, input order, attrs, outputs      custom_helper_op/cc/ops/custom_helper_ops.cc:190-307
+//   op names, input order, attrs, outputs      custom_helper_op/cc/ops/custom_helper_ops.cc:190-307,
+//                                               :374-411 (CostAggregate, CostAggregateGrad)
 //   output shapes [B,H,W,D,C|groups], mask      custom_helper_ops.cc:214-219, :281-286
 //   validation messages and InvalidArgument     cost_volume_kernels.cc:91-106, :220-243;
 //                                               cost_volume_kernels_v2.cc:93-110, :221-247
@@ -122,6 +123,47 @@ REGISTER_OP("CostVolumeGradV2")
     .Output("base_plane_grad: dtype")
     .SetShapeFn(GradShapes);
 
+// cost and cost_mask [B,H,W,D] (CostAggregateShapeFn, custom_helper_ops.cc:46-58)
+REGISTER_OP("CostAggregate")
+    .Input("ref_image: dtype")
+    .Input("src_images: dtype")
+    .Input("base_plane: dtype")
+    .Input("offsets: dtype")
+    .Input("rs: dtype")
+    .Input("ts: dtype")
+    .Attr("dtype: {float32,float64}")
+    .Attr("reduce_method: string")
+    .Attr("half_centor: bool")
+    .Output("cost: dtype")
+    .Output("cost_mask: int32")
+    .SetShapeFn([](InferenceContext* c) {
+      ShapeHandle ref, offsets;
+      TF_RETURN_IF_ERROR(c->WithRank(c->input(0), 4, &ref));
+      TF_RETURN_IF_ERROR(c->WithRank(c->input(3), 2, &offsets));
+      const ShapeHandle out =
+          c->MakeShape({c->Dim(ref, 0), c->Dim(ref, 1), c->Dim(ref, 2), c->Dim(offsets, 1)});
+      c->set_output(0, out);
+      c->set_output(1, out);
+      return Status::OK();
+    });
+
+REGISTER_OP("CostAggregateGrad")
+    .Input("ref_image: dtype")
+    .Input("src_images: dtype")
+    .Input("base_plane: dtype")
+    .Input("offsets: dtype")
+    .Input("rs: dtype")
+    .Input("ts: dtype")
+    .Input("cost_grad: dtype")
+    .Input("cost_mask: int32")
+    .Attr("dtype: {float32,float64}")
+    .Attr("reduce_method: string")
+    .Attr("half_centor: bool")
+    .Output("ref_image_grad: dtype")
+    .Output("src_images_grad: dtype")
+    .Output("base_plane_grad: dtype")
+    .SetShapeFn(GradShapes);
+
 #if GOOGLE_CUDA || TENSORFLOW_USE_ROCM
 
 typedef Eigen::GpuDevice GPUDevice;
@@ -152,6 +194,30 @@ inline int Bwd(void* s, int r, int h, const int64* d, const double* a, const dou
                const double* cg, const int32* m, double* o0, double* o1, double* o2) {
   return chop_cost_volume_bwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b, c,
                                   e, f, g, cg, m, o0, o1, o2);
+}
+inline int FwdAgg(void* s, int r, int h, const int64* d, const float* a, const float* b,
+                  const float* c, const float* e, const float* f, const float* g, float* o,
+                  int32* m) {
+  return chop_cost_aggregate_fwd_f32(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b,
+                                     c, e, f, g, o, m);
+}
+inline int FwdAgg(void* s, int r, int h, const int64* d, const double* a, const double* b,
+                  const double* c, const double* e, const double* f, const double* g, double* o,
+                  int32* m) {
+  return chop_cost_aggregate_fwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b,
+                                     c, e, f, g, o, m);
+}
+inline int BwdAgg(void* s, int r, int h, const int64* d, const float* a, const float* b,
+                  const float* c, const float* e, const float* f, const float* g, const float* cg,
+                  const int32* m, float* o0, float* o1, float* o2) {
+  return chop_cost_aggregate_bwd_f32(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b,
+                                     c, e, f, g, cg, m, o0, o1, o2);
+}
+inline int BwdAgg(void* s, int r, int h, const int64* d, const double* a, const double* b,
+                  const double* c, const double* e, const double* f, const double* g,
+                  const double* cg, const int32* m, double* o0, double* o1, double* o2) {
+  return chop_cost_aggregate_bwd_f64(s, r, h, d[0], d[1], d[2], d[3], d[4], d[5], d[6], d[7], a, b,
+                                     c, e, f, g, cg, m, o0, o1, o2);
 }
 inline int FwdV2(void* s, int r, int h, const int64* d, int groups, const float* a, const float* b,
                  const float* c, const float* f, const float* g, float* o, int32* m) {
@@ -371,6 +437,68 @@ class CostVolumeGradV2Op : public OpKernel {
   Attrs attrs_;
 };
 
+// CostAggregateOp / CostAggregateGradOp (cost_aggregate_kernels.cc:58-131, :163-259)
+template <typename T>
+class CostAggregateOp : public OpKernel {
+ public:
+  explicit CostAggregateOp(OpKernelConstruction* ctx) : OpKernel(ctx) { attrs_.Read(ctx, false); }
+  void Compute(OpKernelContext* ctx) override {
+    const Tensor &ref = ctx->input(0), &src = ctx->input(1), &plane = ctx->input(2),
+                 &offsets = ctx->input(3), &rs = ctx->input(4), &ts = ctx->input(5);
+    Shapes s;
+    OP_REQUIRES_OK(ctx, s.Check(ref, src, rs, ts));
+    OP_REQUIRES_OK(ctx, s.CheckPlane(plane, offsets));
+    const int64 *d = s.dims;
+    const TensorShape out({d[0], d[1], d[2], d[4]});
+    Tensor *cost = nullptr, *mask = nullptr;
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(0, out, &cost));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(1, out, &mask));
+    OP_REQUIRES_OK(ctx, FromChop(FwdAgg(StreamOf(ctx), attrs_.reduce, attrs_.half_centor, d,
+                                        ref.flat<T>().data(), src.flat<T>().data(),
+                                        plane.flat<T>().data(), offsets.flat<T>().data(),
+                                        rs.flat<T>().data(), ts.flat<T>().data(),
+                                        cost->flat<T>().data(), mask->flat<int32>().data())));
+  }
+
+ private:
+  Attrs attrs_;
+};
+
+template <typename T>
+class CostAggregateGradOp : public OpKernel {
+ public:
+  explicit CostAggregateGradOp(OpKernelConstruction* ctx) : OpKernel(ctx) {
+    attrs_.Read(ctx, false);
+  }
+  void Compute(OpKernelContext* ctx) override {
+    const Tensor &ref = ctx->input(0), &src = ctx->input(1), &plane = ctx->input(2),
+                 &offsets = ctx->input(3), &rs = ctx->input(4), &ts = ctx->input(5),
+                 &cost_grad = ctx->input(6), &cost_mask = ctx->input(7);
+    Shapes s;
+    OP_REQUIRES_OK(ctx, s.Check(ref, src, rs, ts));
+    OP_REQUIRES_OK(ctx, s.CheckPlane(plane, offsets));
+    const TensorShape want({s.dims[0], s.dims[1], s.dims[2], s.dims[4]});
+    OP_REQUIRES(ctx, cost_grad.shape() == want,
+                errors::InvalidArgument("cost_grad must have rank 4, and must compate to ref_image"));
+    OP_REQUIRES(ctx, cost_mask.shape() == want,
+                errors::InvalidArgument("cost_mask must have rank 4, and must compate to ref_image"));
+    Tensor *g0 = nullptr, *g1 = nullptr, *g2 = nullptr;
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(0, ref.shape(), &g0));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(1, src.shape(), &g1));
+    OP_REQUIRES_OK(ctx, ctx->allocate_output(2, plane.shape(), &g2));
+    OP_REQUIRES_OK(ctx, FromChop(BwdAgg(StreamOf(ctx), attrs_.reduce, attrs_.half_centor, s.dims,
+                                        ref.flat<T>().data(), src.flat<T>().data(),
+                                        plane.flat<T>().data(), offsets.flat<T>().data(),
+                                        rs.flat<T>().data(), ts.flat<T>().data(),
+                                        cost_grad.flat<T>().data(), cost_mask.flat<int32>().data(),
+                                        g0->flat<T>().data(), g1->flat<T>().data(),
+                                        g2->flat<T>().data())));
+  }
+
+ private:
+  Attrs attrs_;
+};
+
 #define REGISTER_CHOP(NAME, CLASS, TYPE) \
   REGISTER_KERNEL_BUILDER(Name(NAME).Device(DEVICE_GPU).TypeConstraint<TYPE>("dtype"), CLASS<TYPE>)
 
@@ -382,6 +510,10 @@ REGISTER_CHOP("CostVolumeV2", CostVolumeV2Op, float);
 REGISTER_CHOP("CostVolumeV2", CostVolumeV2Op, double);
 REGISTER_CHOP("CostVolumeGradV2", CostVolumeGradV2Op, float);
 REGISTER_CHOP("CostVolumeGradV2", CostVolumeGradV2Op, double);
+REGISTER_CHOP("CostAggregate", CostAggregateOp, float);
+REGISTER_CHOP("CostAggregate", CostAggregateOp, double);
+REGISTER_CHOP("CostAggregateGrad", CostAggregateGradOp, float);
+REGISTER_CHOP("CostAggregateGrad", CostAggregateGradOp, double);
 
 #undef REGISTER_CHOP
 

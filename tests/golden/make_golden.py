@@ -2,7 +2,7 @@
 
 The reference holds no vectors for this path and cannot be run here (TensorFlow + CUDA), so
 these fixtures are produced by this repository's oracle AFTER it passed the pinning tests
-(tests/test_oracle_forward.py, tests/test_oracle_backward.py).  They freeze its behaviour:
+(tests/test_oracle_forward.py, tests/test_oracle_backward.py, tests/test_oracle_aggregate.py).  They freeze its behaviour:
 the CPU suite checks that the oracle still reproduces them bit for bit, the GPU suite checks
 the HIP library against them.  Run from the repository root:
     python tests/golden/make_golden.py
@@ -39,6 +39,13 @@ def cases():
     out["v1_bench2_nohalf_MEAN_f32"] = ("v1", "MEAN", 1, False, wl.tensors)
     wl = make_workload(4, hw=(8, 12), batch=1)
     out["v2_bench4_MEAN_f32"] = ("v2", "MEAN", 4, True, wl.tensors)
+    # CostAggregate (appended last: the cases above keep their random upstream gradients)
+    for dt, tag in ((np.float64, "f64"), (np.float32, "f32")):
+        t = reference_test_case(3, 1, 2, 8, 12, 8, 4, dt, seed=11)
+        for red in ("MEAN", "MIN"):
+            out["agg_ref3_%s_%s" % (red, tag)] = ("agg", red, 1, True, t)
+    wl = make_workload(2, hw=(6, 8), depth=8)
+    out["agg_bench2_MEAN_f32"] = ("agg", "MEAN", 1, True, wl.tensors)
     return out
 
 
@@ -47,6 +54,10 @@ def run(op, red, groups, half, t, cost_grad):
         a = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
         cost, mask = oracle.cost_volume_fwd(*a, red, half)
         grads = oracle.cost_volume_bwd(*a, cost_grad(cost), mask, red, half)
+    elif op == "agg":
+        a = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+        cost, mask = oracle.cost_aggregate_fwd(*a, red, half)
+        grads = oracle.cost_aggregate_bwd(*a, cost_grad(cost), mask, red, half)
     else:
         a = (t["ref"], t["src"], t["depth_grid"], t["Rs"], t["Ts"])
         cost, mask = oracle.cost_volume_v2_fwd(*a, red, groups, half)
@@ -65,11 +76,11 @@ def main():
             return cg_holder["cg"]
 
         cost, mask, grads = run(op, red, groups, half, t, cost_grad)
-        keys = ("ref", "src", "Rs", "Ts") + (("base_plane", "offsets") if op == "v1" else ("depth_grid",))
+        keys = ("ref", "src", "Rs", "Ts") + (("depth_grid",) if op == "v2" else ("base_plane", "offsets"))
         for k in keys:
             blob[name + "/in/" + k] = t[k]
         blob[name + "/in/cost_grad"] = cg_holder["cg"]
-        blob[name + "/attrs"] = np.array([0 if op == "v1" else 1, 0 if red == "MEAN" else 1, groups,
+        blob[name + "/attrs"] = np.array([{"v1": 0, "v2": 1, "agg": 2}[op], 0 if red == "MEAN" else 1, groups,
                                           int(half)], np.int64)
         blob[name + "/out/cost"] = cost
         blob[name + "/out/mask"] = mask

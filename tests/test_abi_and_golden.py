@@ -127,7 +127,7 @@ def _golden_cases():
 
 def test_oracle_reproduces_golden_vectors(oracle):
     blob, names = _golden_cases()
-    assert len(names) == 15
+    assert len(names) == 20
     for name in names:
         op, red, groups, half = (int(x) for x in blob[name + "/attrs"])
         t = {k.split("/")[-1]: blob[k] for k in blob.files if k.startswith(name + "/in/")}
@@ -136,6 +136,10 @@ def test_oracle_reproduces_golden_vectors(oracle):
             a = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
             cost, mask = oracle.cost_volume_fwd(*a, red_s, bool(half))
             grads = oracle.cost_volume_bwd(*a, t["cost_grad"], mask, red_s, bool(half))
+        elif op == 2:
+            a = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+            cost, mask = oracle.cost_aggregate_fwd(*a, red_s, bool(half))
+            grads = oracle.cost_aggregate_bwd(*a, t["cost_grad"], mask, red_s, bool(half))
         else:
             a = (t["ref"], t["src"], t["depth_grid"], t["Rs"], t["Ts"])
             cost, mask = oracle.cost_volume_v2_fwd(*a, red_s, groups, bool(half))

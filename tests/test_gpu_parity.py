@@ -341,6 +341,11 @@ def test_golden_vectors(family):
             ins = [dev(t[k]) for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts")]
             cost, mask = chop.cost_volume_raw(*ins, red_s, bool(half))
             got = chop.cost_volume_grad(*ins, dev(t["cost_grad"]), dev(want_mask), red_s, bool(half))
+        elif op == 2:
+            ins = [dev(t[k]) for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts")]
+            cost, mask = chop.cost_aggregate_raw(*ins, red_s, bool(half))
+            got = chop.cost_aggregate_grad(*ins, dev(t["cost_grad"]), dev(want_mask), red_s,
+                                           bool(half))
         else:
             ins = [dev(t[k]) for k in ("ref", "src", "depth_grid", "Rs", "Ts")]
             cost, mask = chop.cost_volume_v2_raw(*ins, red_s, groups, bool(half))
@@ -350,7 +355,7 @@ def test_golden_vectors(family):
         if family == 1:
             assert np.array_equal(host(cost), want_cost), name
         else:
-            assert_forward_close(host(cost), want_cost, atol=1e-5 if op else 1e-6)
+            assert_forward_close(host(cost), want_cost, atol=1e-5 if op == 1 else 1e-6)
         tol = 1e-4 if want_cost.dtype == np.float32 else 1e-10
         for g, k in zip(got, ("ref_grad", "src_grad", "depth_grad")):
             assert_backward_close(host(g), blob[name + "/out/" + k], tol)
