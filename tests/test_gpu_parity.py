@@ -425,3 +425,55 @@ def test_large_batch_stress_full_size():
     for a1, a2 in zip(g1, g2):
         scale = float(a1.abs().max())
         assert float((a2 - 2 * a1).abs().max()) <= 2e-4 * scale
+
+
+# ---- every lanes-per-pixel variant of the tiled kernels -------------------------------------
+@pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
+@pytest.mark.parametrize("N", [1, 3])
+def test_tiled_channel_widths(oracle, C, N):
+    """C = 4, 8, 16, 32, 64 select 1, 2, 4, 8 and 16 lanes per pixel, each with its own record
+    path, window size and prefetch depth; D = 21 leaves a partial last chunk everywhere."""
+    B, H, W, D = 2, 20, 24, 21
+    rng = np.random.default_rng(C + N)
+    for case in (1, 3):
+        t = reference_test_case(case, B, N, H, W, C, D, np.float32, seed=100 + case)
+        args = tuple(t[k] for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts"))
+        want_cost, want_mask = oracle.cost_volume_fwd(*args)
+        cost, mask = chop.cost_volume_raw(*_v1_inputs(t))
+        _assert_family(0)
+        assert np.array_equal(host(mask), want_mask)
+        assert_forward_close(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+        want = oracle.cost_volume_bwd(*args, cg, want_mask)
+        got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), dev(want_mask))
+        _assert_family(0)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+        # group correlation with per-voxel depths on the same tensors
+        groups = C // 2
+        grid = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(np.float32)
+        a2 = (t["ref"], t["src"], grid, t["Rs"], t["Ts"])
+        want_cost, want_mask = oracle.cost_volume_v2_fwd(*a2, "MEAN", groups)
+        ins = [dev(x) for x in a2]
+        cost, mask = chop.cost_volume_v2_raw(*ins, "MEAN", groups)
+        _assert_family(0)
+        assert np.array_equal(host(mask), want_mask)
+        assert_forward_close(host(cost), want_cost, atol=1e-5)
+        cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+        want = oracle.cost_volume_v2_bwd(*a2, cg, want_mask, "MEAN", groups)
+        got = chop.cost_volume_grad_v2(*ins, dev(cg), dev(want_mask), "MEAN", groups)
+        _assert_family(0)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+        # summed squared difference
+        want_cost, want_mask = oracle.cost_aggregate_fwd(*args)
+        cost, mask = chop.cost_aggregate_raw(*_v1_inputs(t))
+        _assert_family(0)
+        assert np.array_equal(host(mask), want_mask)
+        assert_forward_close(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+        want = oracle.cost_aggregate_bwd(*args, cg, want_mask)
+        got = chop.cost_aggregate_grad(*_v1_inputs(t), dev(cg), dev(want_mask))
+        _assert_family(0)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
