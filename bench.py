@@ -4,6 +4,10 @@ A step is one forward + one backward of the operator (through the C ABI) on one 
 synthetic input that is already resident in HBM.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2] [--no-cpu-baseline]
+
+The default run is the headline configuration (workload 2, MEAN).  ``--reduce MIN`` and
+``--aggregate`` (CostAggregate on the same tensors, float32 workloads only) time the other
+entry points for the tables under profiles/.
 """
 import argparse
 import json
@@ -32,13 +36,16 @@ class Runner:
         self.ref, self.src = up("ref", td), up("src", td)
         self.Rs, self.Ts = up("Rs"), up("Ts")
         self.v2 = wl.op == "v2"
+        self.agg = wl.op == "agg"
+        self.red = 0 if wl.reduce_method == "MEAN" else 1
         if self.v2:
             self.depth_grid = up("depth_grid")
         else:
             self.base_plane, self.offsets = up("base_plane"), up("offsets")
         B, H, W, D, OC = wl.B, wl.H, wl.W, wl.D, wl.out_channels
         self.cost = torch.empty((B, H, W, D, OC), dtype=td, device=d)
-        self.mask = torch.empty((B, H, W, D, 1), dtype=torch.int32, device=d)
+        self.mask = torch.empty((B, H, W, D, 1 if self.red == 0 else OC), dtype=torch.int32,
+                                device=d)
         gen = torch.Generator(device=d)
         gen.manual_seed(wl.seed)
         self.cost_grad = torch.randn((B, H, W, D, OC), dtype=torch.float32, device=d,
@@ -60,21 +67,25 @@ class Runner:
         lib, s = self.lib, self.stream
         if self.v2:
             if self.storage_code:
-                rc = lib.chop_cost_volume_v2_fwd_16(s, self.storage_code, 0, 1, *self.dims,
+                rc = lib.chop_cost_volume_v2_fwd_16(s, self.storage_code, self.red, 1, *self.dims,
                                                     self.wl.groups, p(self.ref), p(self.src),
                                                     p(self.depth_grid), p(self.Rs), p(self.Ts),
                                                     p(self.cost), p(self.mask))
             else:
-                rc = lib.chop_cost_volume_v2_fwd_f32(s, 0, 1, *self.dims, self.wl.groups,
+                rc = lib.chop_cost_volume_v2_fwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
                                                      p(self.ref), p(self.src), p(self.depth_grid),
                                                      p(self.Rs), p(self.Ts), p(self.cost),
                                                      p(self.mask))
+        elif self.agg:
+            rc = lib.chop_cost_aggregate_fwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
+                                                 p(self.base_plane), p(self.offsets), p(self.Rs),
+                                                 p(self.Ts), p(self.cost), p(self.mask))
         elif self.storage_code:
-            rc = lib.chop_cost_volume_fwd_16(s, self.storage_code, 0, 1, *self.dims, p(self.ref),
+            rc = lib.chop_cost_volume_fwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
                                              p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
         else:
-            rc = lib.chop_cost_volume_fwd_f32(s, 0, 1, *self.dims, p(self.ref), p(self.src),
+            rc = lib.chop_cost_volume_fwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
                                               p(self.base_plane), p(self.offsets), p(self.Rs),
                                               p(self.Ts), p(self.cost), p(self.mask))
         if rc:
@@ -87,21 +98,25 @@ class Runner:
                 p(self.depth_grad))
         if self.v2:
             if self.storage_code:
-                rc = lib.chop_cost_volume_v2_bwd_16(s, self.storage_code, 0, 1, *self.dims,
+                rc = lib.chop_cost_volume_v2_bwd_16(s, self.storage_code, self.red, 1, *self.dims,
                                                     self.wl.groups, p(self.ref), p(self.src),
                                                     p(self.depth_grid), p(self.Rs), p(self.Ts),
                                                     *tail, p(self.ws), self.ws_bytes)
             else:
-                rc = lib.chop_cost_volume_v2_bwd_f32(s, 0, 1, *self.dims, self.wl.groups,
+                rc = lib.chop_cost_volume_v2_bwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
                                                      p(self.ref), p(self.src), p(self.depth_grid),
                                                      p(self.Rs), p(self.Ts), *tail)
+        elif self.agg:
+            rc = lib.chop_cost_aggregate_bwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
+                                                 p(self.base_plane), p(self.offsets), p(self.Rs),
+                                                 p(self.Ts), *tail)
         elif self.storage_code:
-            rc = lib.chop_cost_volume_bwd_16(s, self.storage_code, 0, 1, *self.dims, p(self.ref),
+            rc = lib.chop_cost_volume_bwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
                                              p(self.Rs), p(self.Ts), *tail, p(self.ws),
                                              self.ws_bytes)
         else:
-            rc = lib.chop_cost_volume_bwd_f32(s, 0, 1, *self.dims, p(self.ref), p(self.src),
+            rc = lib.chop_cost_volume_bwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
                                               p(self.base_plane), p(self.offsets), p(self.Rs),
                                               p(self.Ts), *tail)
         if rc:
@@ -133,13 +148,18 @@ def cpu_baseline(wl, budget_s=12.0):
         if wl.op == "v1":
             bp = t["base_plane"][:, sl]
             args = (ref, src, bp, t["offsets"], t["Rs"], t["Ts"])
-            _, mask = oracle.cost_volume_fwd(*args, threads=threads)
-            oracle.cost_volume_bwd(*args, cg, mask, threads=threads)
+            _, mask = oracle.cost_volume_fwd(*args, wl.reduce_method, threads=threads)
+            oracle.cost_volume_bwd(*args, cg, mask, wl.reduce_method, threads=threads)
+        elif wl.op == "agg":
+            bp = t["base_plane"][:, sl]
+            args = (ref, src, bp, t["offsets"], t["Rs"], t["Ts"])
+            _, mask = oracle.cost_aggregate_fwd(*args, wl.reduce_method, threads=threads)
+            oracle.cost_aggregate_bwd(*args, cg[..., 0], mask, wl.reduce_method, threads=threads)
         else:
             dg = t["depth_grid"][:, sl]
             args = (ref, src, dg, t["Rs"], t["Ts"])
-            _, mask = oracle.cost_volume_v2_fwd(*args, "MEAN", wl.groups, threads=threads)
-            oracle.cost_volume_v2_bwd(*args, cg, mask, "MEAN", wl.groups, threads=threads)
+            _, mask = oracle.cost_volume_v2_fwd(*args, wl.reduce_method, wl.groups, threads=threads)
+            oracle.cost_volume_v2_bwd(*args, cg, mask, wl.reduce_method, wl.groups, threads=threads)
         times.append(time.perf_counter() - t0)
         if sum(times) > budget_s:
             break
@@ -158,6 +178,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--reduce", choices=["MEAN", "MIN"], default="MEAN")
+    ap.add_argument("--aggregate", action="store_true",
+                    help="time CostAggregate on the workload's tensors (float32 CostVolume workloads)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
@@ -170,6 +193,11 @@ def main():
     from custom_helper_op_amd.configs import make_workload
     lib = _lib.load()
     wl = make_workload(a.workload, with_cost_grad=False)
+    wl.reduce_method = a.reduce
+    if a.aggregate:
+        if wl.op != "v1" or wl.storage != "f32":
+            sys.exit("bench.py: --aggregate needs a float32 CostVolume workload (1, 2 or 5)")
+        wl.op = "agg"
     r = Runner(wl, torch, lib)
     ev = lambda: torch.cuda.Event(enable_timing=True)
     for _ in range(a.warmup):
@@ -206,7 +234,7 @@ def main():
     traffic = None
     try:  # measured with rocprofv3 counters in a separate run; the summary is under profiles/
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            t = json.load(f)[wl.name][dominant]
+            t = json.load(f)[wl.name if wl.op != "agg" and a.reduce == "MEAN" else "-"][dominant]
         traffic = t["fetch_bytes"] + t["write_bytes"]
     except (OSError, KeyError, ValueError):
         pass
@@ -218,9 +246,10 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": wl.storage, "data": "synthetic",
         "config": {"workload": "%s: %s B%d N%d %dx%d C%d D%d%s %s fwd+bwd" % (
-            wl.name, "CostVolume" if wl.op == "v1" else "CostVolumeV2", wl.B, wl.N, wl.H, wl.W,
+            wl.name, {"v1": "CostVolume", "v2": "CostVolumeV2", "agg": "CostAggregate"}[wl.op],
+            wl.B, wl.N, wl.H, wl.W,
             wl.C, wl.D, " G%d" % wl.groups if wl.op == "v2" else "", wl.storage),
-            "voxels": wl.voxels, "reduce_method": "MEAN", "half_centor": True},
+            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic,

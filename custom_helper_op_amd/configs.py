@@ -22,6 +22,7 @@ class Workload:
     name: str
     op: str                # "v1": CostVolume (base_plane + offsets, squared difference)
                            # "v2": CostVolumeV2 (depth_grid, group-wise correlation)
+                           # "agg": CostAggregate (v1's inputs, channels summed: one value/voxel)
     storage: str           # element type of ref/src/cost/cost_grad: f32, f64, f16, bf16
     B: int
     N: int
@@ -42,7 +43,7 @@ class Workload:
 
     @property
     def out_channels(self) -> int:
-        return self.groups if self.op == "v2" else self.C
+        return self.groups if self.op == "v2" else 1 if self.op == "agg" else self.C
 
     def elem_bytes(self) -> int:
         return {"f32": 4, "f64": 8, "f16": 2, "bf16": 2}[self.storage]
@@ -59,7 +60,7 @@ class Workload:
         ref = px * self.C * e
         src = self.B * self.N * self.H * self.W * self.C * e
         cams = self.B * self.N * 12 * f
-        if self.op == "v1":
+        if self.op != "v2":
             depth_in = px * f + self.B * self.D * f
             depth_grad = px * f
         else:
@@ -67,6 +68,8 @@ class Workload:
             depth_grad = px * self.D * f
         cost = self.voxels * self.out_channels * e
         mask = self.voxels * 4 * (1 if self.reduce_method == "MEAN" else self.out_channels)
+        if self.op == "agg":
+            cost = self.voxels * e  # one value per voxel
         fwd = ref + src + depth_in + cams + cost + mask
         bwd = ref + src + depth_in + cams + cost + mask + ref + src + depth_grad
         return fwd, bwd

@@ -349,12 +349,32 @@ __device__ __forceinline__ float voxel_depth(const Args<S> &a, int64_t pix, int 
 // =========================================================================================
 // Forward
 // =========================================================================================
+// Stores CNT (1, 2 or 4) consecutive int32 values, non-temporal.
+template <int CNT>
+__device__ __forceinline__ void store_ints(int32_t *p, const int *v) {
+  if constexpr (CNT == 4) {
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    i32x4 w = {v[0], v[1], v[2], v[3]};
+    __builtin_nontemporal_store(w, reinterpret_cast<i32x4 *>(p));
+  } else if constexpr (CNT == 2) {
+    typedef int i32x2 __attribute__((ext_vector_type(2)));
+    i32x2 w = {v[0], v[1]};
+    __builtin_nontemporal_store(w, reinterpret_cast<i32x2 *>(p));
+  } else {
+    __builtin_nontemporal_store(v[0], p);
+  }
+}
+
 template <int NV>
 constexpr int forward_lds_words(int lpp) {
   return lpp > 1 ? NV * 64 * 5 : 0;
 }
 
-template <typename S, int VEC, int LPP, int NV, int CORR>
+// REDUCE: 0 mean over the accepted views (mask = their number), 1 per-channel minimum of
+// the squared difference / per-group maximum of the correlation with the winning view as
+// mask (-1: none).  The winner must be the reference's, so that reduce uses the literal
+// operand order with every operation rounded separately instead of the fused chains.
+template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0>
 // At most five waves per SIMD: with six (the two-view instantiation needs only 80 VGPRs)
 // the waves of a CU evict each other's taps from L1 and the kernel is 6 % slower.
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void forward_kernel(
@@ -419,7 +439,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           r_wts[n] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
         }
       }
-      if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
+      if constexpr (REDUCE == 0)
+        if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
     }
     if constexpr (LPP > 1) wave_sync();
     float agg_out = 0.f;
@@ -429,8 +450,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       const int d = d0 + jj;
       if (d >= d_hi) break;
       float acc[VEC];
+      int arg[VEC];  // REDUCE == 1: winning view per channel (or per group)
 #pragma unroll
-      for (int c = 0; c < VEC; ++c) acc[c] = 0.f;
+      for (int c = 0; c < VEC; ++c) {
+        // numeric_limits::max() / ::min() seeds, cost_volume_kernels_gpu.cu.cc:174-177 and
+        // cost_volume_kernels_gpu_v2.cu.cc:179
+        acc[c] = REDUCE == 0 ? 0.f : CORR == 0 ? 3.402823466e+38f : 1.175494351e-38f;
+        arg[c] = -1;
+      }
       int k = 0;
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
@@ -452,6 +479,39 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
             load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
             load_vec<S, VEC, false>(q + row_step, tap[n][3]);
           }
+          if constexpr (REDUCE == 1) {
+            float val[VEC];
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+              const float smp = wt.x * tap[n][0][c] + wt.y * tap[n][1][c] + wt.z * tap[n][2][c] +
+                                wt.w * tap[n][3][c];
+              if (CORR == 0) {
+                const float diff = smp - ref[c];
+                val[c] = diff * diff;
+              } else {
+                val[c] = smp * ref[c];
+              }
+            }
+            if (CORR == 0) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c)
+                if (acc[c] > val[c]) acc[c] = val[c], arg[c] = n;
+            } else {
+              // groups of sub consecutive channels, summed in channel order from zero
+#pragma unroll
+              for (int gi = 0; gi < VEC; ++gi) {
+                if (gi * g.sub < VEC) {
+                  float corr = 0.f;
+#pragma unroll
+                  for (int c = 0; c < VEC; ++c)
+                    if (c >= gi * g.sub && c < (gi + 1) * g.sub) corr += val[c];
+                  if (acc[gi] < corr) acc[gi] = corr, arg[gi] = n;
+                }
+              }
+            }
+            ++k;
+            continue;
+          }
 #pragma unroll
           for (int c = 0; c < VEC; ++c) {
             if (CORR != 1) {
@@ -471,6 +531,22 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           }
           ++k;
         }
+      }
+      if constexpr (REDUCE == 1) {
+        if (t.pix_ok) {
+          S *out = a.cost + (t.pix * D + d) * OC;
+          int32_t *mout = a.mask + (t.pix * D + d) * OC;
+          if (CORR == 0) {
+            store_vec<S, VEC, true>(out + t.cl * VEC, acc);
+            store_ints<VEC>(mout + t.cl * VEC, arg);
+          } else {
+            store_groups<S, VEC, true>(out + t.cl * gv, acc, g.sub);
+            if (g.sub == 1) store_ints<VEC>(mout + t.cl * gv, arg);
+            else if (g.sub == 2) store_ints<VEC / 2>(mout + t.cl * gv, arg);
+            else store_ints<VEC / 4>(mout + t.cl * gv, arg);
+          }
+        }
+        continue;
       }
       if constexpr (CORR == 2) {
         // one value per voxel: the pixel's lanes add up their channels; the lane whose
