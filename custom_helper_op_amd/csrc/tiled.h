@@ -775,7 +775,11 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
 // beats two views at two.
 constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 : nv <= 2 ? 2 : 1; }
 
-template <typename S, int VEC, int LPP, int NV, int CORR>
+// REDUCE: 0 gradient of the mean (mask = number of accepted views), 1 gradient of the
+// per-channel minimum / per-group maximum (mask = winning view per channel or group; a
+// voxel is skipped when its first entry is negative, cost_volume_kernels_gpu.cu.cc:483-486)
+// and of the summed-squared-difference minimum (mask = the voxel's winning view).
+template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0>
 __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
   using WN = Window<VEC, LPP>;
@@ -842,19 +846,23 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
-  constexpr int PF = LPP < 8 ? LPP : 8;  // upstream-gradient rows fetched ahead
+  // upstream-gradient rows fetched ahead; the MIN reduce stages the mask rows beside them
+  constexpr int PFMAX = REDUCE ? 4 : 8;
+  constexpr int PF = LPP < PFMAX ? LPP : PFMAX;
+  constexpr bool kMaskRows = REDUCE == 1 && CORR != 2;
   const S *cg_lane = a.cost_grad + t.pix * D * OC + (CORR == 2 ? 0 : t.cl * (CORR ? gv : VEC));
   const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
-  const int32_t *cnt_src = a.mask_in + t.pix * D;
+  const int32_t *cnt_src = a.mask_in + t.pix * D * (kMaskRows ? OC : 1);
+  const int32_t *mask_lane = cnt_src + t.cl * (CORR ? gv : VEC);  // this lane's part of a mask row
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
     // Depth hypothesis and valid-view count of lane (p, j)'s voxel: requested before the
     // chunk's upstream-gradient rows, because loads return in order and the reprojection
     // should wait for these two words only.
     float dv = 1.f, cg_vox = 0.f;
-    int cnt = 0;
+    int cnt = REDUCE ? -1 : 0;  // "nothing to do" for a lane without a voxel
     if (d0 + t.cl < d_hi) {
       dv = dv_src[d0 + t.cl];
-      if (t.pix_ok) cnt = cnt_src[d0 + t.cl];
+      if (t.pix_ok) cnt = cnt_src[(int64_t)(d0 + t.cl) * (kMaskRows ? OC : 1)];
       if constexpr (CORR == 2)  // the voxel's one upstream gradient rides with its record
         cg_vox = reinterpret_cast<const float *>(cg_lane)[d0 + t.cl];
     }
@@ -867,28 +875,55 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     // next view's workgroup hit L2 more often (690 -> 660 MB fetched) and save 10 us here,
     // but leave the caches full of these rows and cost the next forward launch 25 us.
     float cgr[CORR == 2 ? 1 : PF][VEC];
-    if constexpr (CORR != 2) {
+    int mrow[kMaskRows ? PF : 1][VEC];
+    auto load_rows = [&](int first) {
 #pragma unroll
       for (int jj = 0; jj < PF; ++jj) {
-        const int d = min(d0 + jj, d_hi - 1);
+        const int d = min(first + jj, d_hi - 1);
         const S *src_cg = cg_lane + (int64_t)d * OC;
         if (CORR == 0)
           load_vec<S, VEC, true>(src_cg, cgr[jj]);
         else
           load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
+        if constexpr (kMaskRows) {
+          const int32_t *m = mask_lane + (int64_t)d * OC;
+          const int cntv = CORR == 0 ? VEC : gv;
+          if (cntv == 4) {
+            typedef int i32x4 __attribute__((ext_vector_type(4)));
+            const i32x4 v = __builtin_nontemporal_load(reinterpret_cast<const i32x4 *>(m));
+            mrow[jj][0] = v[0], mrow[jj][1] = v[1], mrow[jj][2] = v[2], mrow[jj][3] = v[3];
+          } else if (cntv == 2) {
+            typedef int i32x2 __attribute__((ext_vector_type(2)));
+            const i32x2 v = __builtin_nontemporal_load(reinterpret_cast<const i32x2 *>(m));
+            mrow[jj][0] = v[0], mrow[jj][1] = v[1];
+          } else {
+            mrow[jj][0] = __builtin_nontemporal_load(m);
+          }
+        }
       }
-    }
+    };
+    if constexpr (CORR != 2) load_rows(d0);
     {
       const float depth = d0 + t.cl < d_hi ? (per_voxel_depth ? dv : base + dv) : 1.f;
       // factor the reduce applies to the upstream gradient: squared difference 2/k,
       // correlation 1/k, summed squared difference 2*cost_grad/(k*C) (the whole per-voxel
       // factor); zero marks a voxel that contributes nothing
       float scl = 0.f;
-      if (cnt > 0) {
-        if constexpr (CORR == 2)
-          scl = 2.f * (cg_vox / static_cast<float>(cnt * C));
-        else
-          scl = (CORR == 0 ? 2.f : 1.f) * __builtin_amdgcn_rcpf(static_cast<float>(cnt));
+      if constexpr (REDUCE == 0) {
+        if (cnt > 0) {
+          if constexpr (CORR == 2)
+            scl = 2.f * (cg_vox / static_cast<float>(cnt * C));
+          else
+            scl = (CORR == 0 ? 2.f : 1.f) * __builtin_amdgcn_rcpf(static_cast<float>(cnt));
+        }
+      } else {
+        // no division by the view count; `cnt` holds the first mask entry of the voxel (or,
+        // for the summed squared difference, its winning view)
+        if constexpr (CORR == 2) {
+          if (cnt == t.view0) scl = 2.f * (cg_vox / static_cast<float>(C));
+        } else {
+          if (cnt >= 0) scl = CORR == 0 ? 2.f : 1.f;
+        }
       }
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
@@ -897,7 +932,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         hit.key = 0;
         hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
         float4 dw4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (t.view0 + n < N && cnt > 0) {
+        if (t.view0 + n < N && scl != 0.f) {
           reproject<NV>(cam, n, depth, half, g.src_h_max, g.src_w_max, srcW, C, hit);
           if (hit.off >= 0) {
             // d(sample)/d(depth) = sum over taps of dwt * tap, from
@@ -979,17 +1014,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       const int d = d0 + jj;
       if (d >= d_hi) break;
       if constexpr (LPP > PF && CORR != 2) {
-        if (jj == PF) {  // second half of a 16-deep chunk
-#pragma unroll
-          for (int j2 = 0; j2 < PF; ++j2) {
-            const int dd = min(d0 + PF + j2, d_hi - 1);
-            const S *src_cg = cg_lane + (int64_t)dd * OC;
-            if (CORR == 0)
-              load_vec<S, VEC, true>(src_cg, cgr[j2]);
-            else
-              load_groups<S, VEC, true>(src_cg, cgr[j2], g.sub);
-          }
-        }
+        if (jj > 0 && jj % PF == 0) load_rows(d0 + jj);  // next part of a deep chunk
       }
       // The records of the NEXT depth are requested now, so that their LDS latency overlaps
       // this depth's arithmetic (jj is unrolled: the buffer index is a compile-time constant).
@@ -1028,6 +1053,19 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           } else {
 #pragma unroll
             for (int c = 0; c < VEC; ++c) cg[c] = raw[0] * scl;
+          }
+          if constexpr (kMaskRows) {
+            // only the channels (groups) this view won contribute
+            static_assert(NV == 1, "the MIN gradient runs one view per workgroup");
+            const int *mr = mrow[jj % PF];
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+              const int win = (CORR == 0 || g.sub == 1) ? mr[c]
+                              : g.sub == 2              ? mr[c / 2]
+                              : g.sub == 4              ? mr[c / 4]
+                                                        : mr[0];
+              if (win != t.view0) cg[c] = 0.f;
+            }
           }
         }
 #pragma unroll

@@ -474,10 +474,34 @@ def test_tiled_channel_widths(oracle, C, N):
         cost, mask = chop.cost_volume_raw(*_v1_inputs(t), "MIN")
         _assert_family(0)
         assert np.array_equal(host(mask), want_mask) and np.array_equal(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+        want = oracle.cost_volume_bwd(*args, cg, want_mask, "MIN")
+        got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), dev(want_mask), "MIN")
+        _assert_family(0)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
         want_cost, want_mask = oracle.cost_volume_v2_fwd(*a2, "MIN", groups)
         cost, mask = chop.cost_volume_v2_raw(*ins, "MIN", groups)
         _assert_family(0)
         assert np.array_equal(host(mask), want_mask) and np.array_equal(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+        want = oracle.cost_volume_v2_bwd(*a2, cg, want_mask, "MIN", groups)
+        got = chop.cost_volume_grad_v2(*ins, dev(cg), dev(want_mask), "MIN", groups)
+        _assert_family(0)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+        # minimum of the summed squared difference: forward on the general kernel (the sum
+        # must follow the reference's channel order to name the same winner), backward tiled
+        want_cost, want_mask = oracle.cost_aggregate_fwd(*args, "MIN")
+        cost, mask = chop.cost_aggregate_raw(*_v1_inputs(t), "MIN")
+        _assert_family(1)
+        assert np.array_equal(host(mask), want_mask) and np.array_equal(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+        want = oracle.cost_aggregate_bwd(*args, cg, want_mask, "MIN")
+        got = chop.cost_aggregate_grad(*_v1_inputs(t), dev(cg), dev(want_mask), "MIN")
+        _assert_family(0)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
         # summed squared difference
         want_cost, want_mask = oracle.cost_aggregate_fwd(*args)
         cost, mask = chop.cost_aggregate_raw(*_v1_inputs(t))
