@@ -170,6 +170,99 @@ int backward(void *stream, int reduce, int half_centor, const Dims &d, int group
   return launch_status(launch_general_backward(a, s), "general backward launch");
 }
 
+// CostVolumeV3 (cost_volume_kernels_v3.cc:94-115): the V1 argument checks plus
+// C % groups == 0 and at most kMaxSubChannels channels per group.
+template <typename S>
+int v3_call(void *stream, int reduce, int half_centor, const Dims &d, int groups, const S *ref,
+            const S *src, const S *base_plane, const S *offsets, const S *Rs, const S *Ts,
+            S *cost, int32_t *mask, const S *cost_grad, const int32_t *mask_in, S *ref_grad,
+            S *src_grad, S *base_plane_grad, bool backward) {
+  if (int rc = check_dims(d, reduce, groups, true)) return rc;
+  if (d.C / groups > kMaxSubChannels)
+    return fail(CHOP_ERR_BAD_GROUPS, "CostVolumeV3 holds at most 8 channels per group");
+  const int64_t pixels = d.B * d.H * d.W, voxels = pixels * d.D;
+  const int64_t n_ref = pixels * d.C, n_src = d.B * d.N * d.srcH * d.srcW * d.C;
+  const bool work = voxels > 0 && d.C > 0;
+  if (backward) {
+    if (n_ref == 0 && n_src == 0 && pixels == 0) return CHOP_OK;
+    REQUIRE_PTR(ref_grad, n_ref);
+    REQUIRE_PTR(src_grad, n_src);
+    REQUIRE_PTR(base_plane_grad, pixels);
+  } else {
+    if (voxels == 0) return CHOP_OK;
+    REQUIRE_PTR(cost, voxels);
+    REQUIRE_PTR(mask, voxels);
+  }
+  if (work || !backward) {
+    REQUIRE_PTR(ref, n_ref);
+    REQUIRE_PTR(src, n_src);
+    REQUIRE_PTR(base_plane, pixels);
+    REQUIRE_PTR(offsets, d.B * d.D);
+    REQUIRE_PTR(Rs, d.B * d.N);
+    REQUIRE_PTR(Ts, d.B * d.N);
+    if (backward) {
+      REQUIRE_PTR(cost_grad, voxels);
+      REQUIRE_PTR(mask_in, voxels);
+    }
+  }
+  Args<S> a{};
+  a.B = d.B, a.H = d.H, a.W = d.W, a.C = d.C, a.D = d.D, a.N = d.N, a.srcH = d.srcH, a.srcW = d.srcW;
+  a.groups = groups, a.reduce = reduce, a.corr = BEST_GROUP_PAIR, a.half = half_centor ? S(0.5) : S(0);
+  a.ref = ref, a.src = src, a.base_plane = base_plane, a.offsets = offsets, a.Rs = Rs, a.Ts = Ts;
+  a.cost = cost, a.mask = mask, a.cost_grad = cost_grad, a.mask_in = mask_in;
+  a.ref_grad = ref_grad, a.src_grad = src_grad, a.depth_grad = base_plane_grad;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  g_last_family = 1;
+  if (backward) return launch_status(launch_v3_backward(a, s), "CostVolumeV3 backward launch");
+  return launch_status(launch_v3_forward(a, s), "CostVolumeV3 forward launch");
+}
+
+// FeatureAggregate (feature_aggregate_kernels.cc:69-92): the output grid H x W is
+// base_plane's, the source images have their own size.
+template <typename S>
+int feature_call(void *stream, int half_centor, const Dims &d, const S *src, const S *base_plane,
+                 const S *offsets, const S *Rs, const S *Ts, S *mapped, int32_t *mapped_mask,
+                 const S *mapped_grad, const int32_t *mask_in, S *src_grad, S *base_plane_grad,
+                 bool backward) {
+  if (int rc = check_dims(d, CHOP_REDUCE_MEAN, 1, false)) return rc;
+  int64_t tmp;
+  if (mul_overflows({d.B, d.H, d.W, d.D, d.N, d.C > 0 ? d.C : 1}, &tmp))
+    return fail(CHOP_ERR_BAD_DIMS, "tensor element count overflows");
+  const int64_t pixels = d.B * d.H * d.W, rows = pixels * d.D * d.N;
+  const int64_t n_src = d.B * d.N * d.srcH * d.srcW * d.C;
+  const bool work = rows > 0 && d.C > 0;
+  if (backward) {
+    if (n_src == 0 && pixels == 0) return CHOP_OK;
+    REQUIRE_PTR(src_grad, n_src);
+    REQUIRE_PTR(base_plane_grad, pixels);
+  } else {
+    if (rows == 0) return CHOP_OK;
+    REQUIRE_PTR(mapped, rows * d.C);
+    REQUIRE_PTR(mapped_mask, rows);
+  }
+  if (work || !backward) {
+    REQUIRE_PTR(src, n_src);
+    REQUIRE_PTR(base_plane, pixels);
+    REQUIRE_PTR(offsets, d.B * d.D);
+    REQUIRE_PTR(Rs, d.B * d.N);
+    REQUIRE_PTR(Ts, d.B * d.N);
+    if (backward) {
+      REQUIRE_PTR(mapped_grad, rows * d.C);
+      REQUIRE_PTR(mask_in, rows);
+    }
+  }
+  Args<S> a{};
+  a.B = d.B, a.H = d.H, a.W = d.W, a.C = d.C, a.D = d.D, a.N = d.N, a.srcH = d.srcH, a.srcW = d.srcW;
+  a.groups = 1, a.reduce = CHOP_REDUCE_MEAN, a.corr = WARP_ONLY, a.half = half_centor ? S(0.5) : S(0);
+  a.src = src, a.base_plane = base_plane, a.offsets = offsets, a.Rs = Rs, a.Ts = Ts;
+  a.cost = mapped, a.mask = mapped_mask, a.cost_grad = mapped_grad, a.mask_in = mask_in;
+  a.src_grad = src_grad, a.depth_grad = base_plane_grad;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  g_last_family = 1;
+  if (backward) return launch_status(launch_feature_backward(a, s), "FeatureAggregate backward launch");
+  return launch_status(launch_feature_forward(a, s), "FeatureAggregate forward launch");
+}
+
 }  // namespace
 }  // namespace chop
 
@@ -312,6 +405,50 @@ int chop_cost_volume_v2_bwd_f64(void *stream, int reduce, int half_centor, int64
                           nullptr, nullptr, depth_grid, Rs, Ts, cost_grad, mask, ref_grad,
                           src_grad, depth_grid_grad, true, nullptr, 0);
 }
+
+#define V3_ENTRY(SFX, T)                                                                       \
+  int chop_cost_volume_v3_fwd_##SFX(void *stream, int reduce, int half_centor, int64_t B,      \
+                                    int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,     \
+                                    int64_t srcH, int64_t srcW, int groups, const T *ref,      \
+                                    const T *src, const T *base_plane, const T *offsets,       \
+                                    const T *Rs, const T *Ts, T *cost, int32_t *mask) {        \
+    return v3_call<T>(stream, reduce, half_centor, DIMS, groups, ref, src, base_plane, offsets, \
+                      Rs, Ts, cost, mask, nullptr, nullptr, nullptr, nullptr, nullptr, false);  \
+  }                                                                                            \
+  int chop_cost_volume_v3_bwd_##SFX(void *stream, int reduce, int half_centor, int64_t B,      \
+                                    int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,     \
+                                    int64_t srcH, int64_t srcW, int groups, const T *ref,      \
+                                    const T *src, const T *base_plane, const T *offsets,       \
+                                    const T *Rs, const T *Ts, const T *cost_grad,              \
+                                    const int32_t *mask, T *ref_grad, T *src_grad,             \
+                                    T *base_plane_grad) {                                      \
+    return v3_call<T>(stream, reduce, half_centor, DIMS, groups, ref, src, base_plane, offsets, \
+                      Rs, Ts, nullptr, nullptr, cost_grad, mask, ref_grad, src_grad,            \
+                      base_plane_grad, true);                                                   \
+  }                                                                                            \
+  int chop_feature_aggregate_fwd_##SFX(void *stream, int half_centor, int64_t B, int64_t H,    \
+                                       int64_t W, int64_t C, int64_t D, int64_t N,             \
+                                       int64_t srcH, int64_t srcW, const T *src,               \
+                                       const T *base_plane, const T *offsets, const T *Rs,     \
+                                       const T *Ts, T *mapped_feature, int32_t *mapped_mask) { \
+    return feature_call<T>(stream, half_centor, DIMS, src, base_plane, offsets, Rs, Ts,        \
+                           mapped_feature, mapped_mask, nullptr, nullptr, nullptr, nullptr,    \
+                           false);                                                             \
+  }                                                                                            \
+  int chop_feature_aggregate_bwd_##SFX(void *stream, int half_centor, int64_t B, int64_t H,    \
+                                       int64_t W, int64_t C, int64_t D, int64_t N,             \
+                                       int64_t srcH, int64_t srcW, const T *src,               \
+                                       const T *base_plane, const T *offsets, const T *Rs,     \
+                                       const T *Ts, const T *mapped_feature_grad,              \
+                                       const int32_t *mapped_mask, T *src_grad,                \
+                                       T *base_plane_grad) {                                   \
+    return feature_call<T>(stream, half_centor, DIMS, src, base_plane, offsets, Rs, Ts,        \
+                           nullptr, nullptr, mapped_feature_grad, mapped_mask, src_grad,       \
+                           base_plane_grad, true);                                             \
+  }
+V3_ENTRY(f32, float)
+V3_ENTRY(f64, double)
+#undef V3_ENTRY
 
 size_t chop_cost_volume_bwd16_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C,
                                               int64_t N, int64_t srcH, int64_t srcW) {

@@ -19,30 +19,6 @@ constexpr int kBlock = 256;
 template <typename S>
 struct Is16 : std::integral_constant<bool, sizeof(S) == 2> {};
 
-template <typename R>
-struct Voxel {
-  int64_t i, pix;
-  int b, h, w, d;
-  R depth, ref_w, ref_h;
-};
-
-template <typename S>
-__device__ __forceinline__ Voxel<typename Storage<S>::Real> locate(const Args<S> &a, int64_t i) {
-  using R = typename Storage<S>::Real;
-  Voxel<R> v;
-  v.i = i;
-  v.pix = i / a.D;
-  v.d = (int)(i - v.pix * a.D);
-  const int64_t row = v.pix / a.W;
-  v.w = (int)(v.pix - row * a.W);
-  v.b = (int)(row / a.H);
-  v.h = (int)(row - (int64_t)v.b * a.H);
-  v.depth = a.depth_grid ? a.depth_grid[i] : a.base_plane[v.pix] + a.offsets[(int64_t)v.b * a.D + v.d];
-  v.ref_w = static_cast<R>(v.w) + a.half;
-  v.ref_h = static_cast<R>(v.h) + a.half;
-  return v;
-}
-
 template <typename S, int CORR, int REDUCE>
 __global__ __launch_bounds__(kBlock) void general_forward_kernel(const Args<S> a) {
   using R = typename Storage<S>::Real;

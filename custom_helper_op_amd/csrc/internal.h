@@ -13,7 +13,20 @@ namespace chop {
 //   SQUARED_DIFFERENCE      (sample - ref)^2 per channel              row = C values
 //   GROUP_CORRELATION       sum over a channel group of sample * ref  row = groups values
 //   SUM_SQUARED_DIFFERENCE  (sample - ref)^2 summed over the channels row = 1 value (CostAggregate)
-enum Corr { SQUARED_DIFFERENCE = 0, GROUP_CORRELATION = 1, SUM_SQUARED_DIFFERENCE = 2 };
+//   BEST_GROUP_PAIR         largest correlation of any source group with any reference group
+//                                                                     row = 1 value (CostVolumeV3)
+//   WARP_ONLY               the sample itself, per view               row = N*C values (FeatureAggregate)
+enum Corr {
+  SQUARED_DIFFERENCE = 0,
+  GROUP_CORRELATION = 1,
+  SUM_SQUARED_DIFFERENCE = 2,
+  BEST_GROUP_PAIR = 3,
+  WARP_ONLY = 4
+};
+
+// Channels per group the CostVolumeV3 kernels hold in registers (MAX_SUBCHANNELS_SIZE,
+// custom_helper_op/cc/kernels/cost_volume_v3.h:35).
+constexpr int kMaxSubChannels = 8;
 
 // One call's arguments after validation.  S = storage type of the feature tensors,
 // R = Storage<S>::Real = type of depth inputs, camera matrices, depth gradients.
@@ -43,15 +56,54 @@ struct Args {
   __host__ __device__ int64_t pixels() const { return B * H * W; }
   __host__ __device__ int64_t voxels() const { return B * H * W * D; }
   __host__ __device__ int out_channels() const {
-    return corr == GROUP_CORRELATION ? groups : corr == SUM_SQUARED_DIFFERENCE ? 1 : (int)C;
+    return corr == GROUP_CORRELATION ? groups
+           : corr == SUM_SQUARED_DIFFERENCE || corr == BEST_GROUP_PAIR ? 1
+           : corr == WARP_ONLY ? (int)(N * C)
+                               : (int)C;
   }
 };
+
+// One voxel of the sweep volume: indices, depth hypothesis and reference-pixel coordinates.
+template <typename R>
+struct Voxel {
+  int64_t i, pix;
+  int b, h, w, d;
+  R depth, ref_w, ref_h;
+};
+
+template <typename S>
+__device__ __forceinline__ Voxel<typename Storage<S>::Real> locate(const Args<S> &a, int64_t i) {
+  using R = typename Storage<S>::Real;
+  Voxel<R> v;
+  v.i = i;
+  v.pix = i / a.D;
+  v.d = (int)(i - v.pix * a.D);
+  const int64_t row = v.pix / a.W;
+  v.w = (int)(v.pix - row * a.W);
+  v.b = (int)(row / a.H);
+  v.h = (int)(row - (int64_t)v.b * a.H);
+  v.depth = a.depth_grid ? a.depth_grid[i] : a.base_plane[v.pix] + a.offsets[(int64_t)v.b * a.D + v.d];
+  v.ref_w = static_cast<R>(v.w) + a.half;
+  v.ref_h = static_cast<R>(v.h) + a.half;
+  return v;
+}
 
 // General kernels: any shape, any channel count, both reduces, all storage types.
 template <typename S>
 hipError_t launch_general_forward(const Args<S> &a, hipStream_t stream);
 template <typename S>
 hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream);
+
+// CostVolumeV3 (corr = BEST_GROUP_PAIR) and FeatureAggregate (corr = WARP_ONLY; `ref` unused,
+// `cost` = mapped_feature [B,H,W,D,N,C], `mask` = mapped_mask [B,H,W,D,N]): float and double.
+template <typename S>
+hipError_t launch_v3_forward(const Args<S> &a, hipStream_t stream);
+template <typename S>
+hipError_t launch_v3_backward(const Args<S> &a, hipStream_t stream);
+template <typename S>
+hipError_t launch_feature_forward(const Args<S> &a, hipStream_t stream);
+template <typename S>
+hipError_t launch_feature_backward(const Args<S> &a, hipStream_t stream);
 
 // Tiled kernels: wavefront-per-pixel-tile, depth innermost.  `supported` says whether the
 // shape qualifies; the launchers must only be called when it does.

@@ -1,0 +1,353 @@
+// CostVolumeV3 and FeatureAggregate: general kernels (any shape, float and double).
+//
+// CostVolumeV3 (custom_helper_op/cc/kernels/cost_volume_kernels_gpu_v3.cu.cc:33-261, 376-639):
+// per accepted view the largest dot product between any channel group of the bilinear sample
+// and any channel group of the reference pixel; MEAN averages the views' maxima, MIN keeps the
+// overall maximum and records (view, reference group, source group).  One thread per voxel:
+// the winner of a voxel is an index triple, so the pairs are visited in the reference's order
+// with its strict comparison, every product and sum rounded separately.
+//
+// FeatureAggregate (feature_aggregate_kernels_gpu.cu.cc:33-121, 219-326): the warp alone,
+// mapped_feature[B,H,W,D,N,C] and a 0/1 mask per (voxel, view).  One thread per (voxel, view,
+// channel slice); a slice is 16 bytes when the channel count and the pointers allow.
+#include <type_traits>
+
+#include "internal.h"
+
+namespace chop {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename R>
+struct Taps {
+  const R *t00, *t01, *t11, *t10;
+};
+
+template <typename R>
+__device__ __forceinline__ Taps<R> taps_of(const R *src, const Sample<R> &s, int64_t cam, int C,
+                                           int srcH, int srcW) {
+  Taps<R> t;
+  t.t00 = src + (int64_t)C * (s.fw + (int64_t)srcW * (s.fh + (int64_t)srcH * cam));
+  t.t01 = t.t00 + C;
+  t.t11 = t.t01 + (int64_t)srcW * C;
+  t.t10 = t.t00 + (int64_t)srcW * C;
+  return t;
+}
+
+// Best (source group, reference group) pair of one accepted sample: source group outermost,
+// strict "<", seeded with `seed` (cost_volume_kernels_gpu_v3.cu.cc:113-130, 231-250).
+// gi, gs are left untouched when no pair exceeds the seed.
+template <typename R>
+__device__ __forceinline__ R best_pair(const Sample<R> &s, const Taps<R> &t, const R *ref_px,
+                                       int groups, int sub, R seed, int &gi_out, int &gs_out) {
+  R buf[kMaxSubChannels];
+  R best = seed;
+  for (int gs = 0; gs < groups; ++gs) {
+#pragma unroll
+    for (int k = 0; k < kMaxSubChannels; ++k) {
+      if (k < sub) {
+        const int sc = gs * sub + k;
+        buf[k] = s.k00 * t.t00[sc] + s.k01 * t.t01[sc] + s.k11 * t.t11[sc] + s.k10 * t.t10[sc];
+      }
+    }
+    for (int gi = 0; gi < groups; ++gi) {
+      R tmp = R(0);
+#pragma unroll
+      for (int k = 0; k < kMaxSubChannels; ++k)
+        if (k < sub) tmp += buf[k] * ref_px[gi * sub + k];
+      if (best < tmp) {
+        best = tmp;
+        gi_out = gi;
+        gs_out = gs;
+      }
+    }
+  }
+  return best;
+}
+
+template <typename R, int REDUCE>
+__global__ __launch_bounds__(kBlock) void v3_forward_kernel(const Args<R> a) {
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int groups = a.groups, sub = C / groups;
+  const int64_t total = a.voxels();
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * kBlock) {
+    const Voxel<R> v = locate(a, i);
+    const R *ref_px = a.ref + v.pix * C;
+    R acc = REDUCE == 0 ? R(0) : Limits<R>::min_positive();
+    int used = 0, wn = -1, wgi = -1, wgs = -1;
+    for (int n = 0; n < N; ++n) {
+      Sample<R> s;
+      const int64_t cam = (int64_t)v.b * N + n;
+      project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+      if (s.state != 2) continue;
+      const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
+      int gi = -1, gs = -1;
+      if (REDUCE == 0) {
+        acc += best_pair(s, t, ref_px, groups, sub, Limits<R>::min_positive(), gi, gs);
+        ++used;
+      } else {
+        const R best = best_pair(s, t, ref_px, groups, sub, acc, gi, gs);
+        if (gi >= 0) {
+          acc = best;
+          wn = n, wgi = gi, wgs = gs;
+        }
+      }
+    }
+    if (REDUCE == 0) {
+      a.mask[i] = used;
+      a.cost[i] = used > 0 ? acc / static_cast<R>(used) : R(0);
+    } else {
+      a.mask[i * 3] = wn, a.mask[i * 3 + 1] = wgi, a.mask[i * 3 + 2] = wgs;
+      a.cost[i] = wn >= 0 ? acc : R(0);
+    }
+  }
+}
+
+template <typename R, int REDUCE>
+__global__ __launch_bounds__(kBlock) void v3_backward_kernel(const Args<R> a) {
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int groups = a.groups, sub = C / groups;
+  const int64_t total = a.voxels();
+  const int64_t row_step = (int64_t)srcW * C;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * kBlock) {
+    const int32_t *m = a.mask_in + (REDUCE == 0 ? i : i * 3);
+    const int32_t m0 = m[0];
+    if (REDUCE == 0 ? (m0 <= 0) : (m0 < 0)) continue;
+    const Voxel<R> v = locate(a, i);
+    const R *ref_px = a.ref + v.pix * C;
+    R *ref_out = a.ref_grad + v.pix * C;
+    // :426 cost_grad / (T)mask for the mean; the MIN gradient takes cost_grad as is (:621)
+    const R cg = REDUCE == 0 ? a.cost_grad[i] / static_cast<R>(m0) : a.cost_grad[i];
+    R depth_grad = R(0);
+    const int n_lo = REDUCE == 0 ? 0 : m0, n_hi = REDUCE == 0 ? N : m0 + 1;
+    for (int n = n_lo; n < n_hi && n < N; ++n) {
+      Sample<R> s;
+      const int64_t cam = (int64_t)v.b * N + n;
+      project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+      // A winner that is not accepted any more (inputs changed since the forward pass) is
+      // skipped; the reference would read and write out of bounds (:593-595).
+      if (s.state != 2) continue;
+      const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
+      int gi = -1, gs = -1;
+      if (REDUCE == 0) {
+        best_pair(s, t, ref_px, groups, sub, Limits<R>::min_positive(), gi, gs);
+        // no pair above the seed: the reference indexes group -1 here (:495-496)
+        if (gi < 0) continue;
+      } else {
+        gi = m[1], gs = m[2];
+        if (gi < 0 || gi >= groups || gs < 0 || gs >= groups) continue;
+      }
+      R *g00 = a.src_grad + (t.t00 - a.src);
+      R h_grad = R(0), w_grad = R(0);
+      for (int k = 0; k < sub; ++k) {
+        const int rc = gi * sub + k, cc = gs * sub + k;
+        const R v00 = t.t00[cc], v01 = t.t01[cc], v11 = t.t11[cc], v10 = t.t10[cc];
+        const R smp = s.k00 * v00 + s.k01 * v01 + s.k11 * v11 + s.k10 * v10;
+        atomic_add(ref_out + rc, cg * smp);
+        const R bg = cg * ref_px[rc];
+        atomic_add(g00 + cc, bg * s.k00);
+        atomic_add(g00 + C + cc, bg * s.k01);
+        atomic_add(g00 + C + row_step + cc, bg * s.k11);
+        atomic_add(g00 + row_step + cc, bg * s.k10);
+        const R t1 = v11 - v10 - v01 + v00;
+        h_grad += bg * (t1 * s.dw + v10 - v00);
+        w_grad += bg * (t1 * s.dh + v01 - v00);
+      }
+      depth_grad += depth_chain(s, h_grad, w_grad);
+    }
+    atomic_add(a.depth_grad + v.pix, depth_grad);
+  }
+}
+
+// ---- FeatureAggregate --------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename R, int VEC>
+struct Slice {
+  R v[VEC];
+};
+
+template <typename R, int VEC>
+__device__ __forceinline__ Slice<R, VEC> load_slice(const R *p) {
+  Slice<R, VEC> out;
+  if constexpr (VEC * sizeof(R) == 16) {
+    const u32x4 raw = *reinterpret_cast<const u32x4 *>(p);
+    __builtin_memcpy(out.v, &raw, 16);
+  } else {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) out.v[k] = p[k];
+  }
+  return out;
+}
+
+template <typename R, int VEC>
+__device__ __forceinline__ void store_slice(R *p, const Slice<R, VEC> &in) {
+  if constexpr (VEC * sizeof(R) == 16) {
+    u32x4 raw;
+    __builtin_memcpy(&raw, in.v, 16);
+    __builtin_nontemporal_store(raw, reinterpret_cast<u32x4 *>(p));  // written once, never re-read
+  } else {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) p[k] = in.v[k];
+  }
+}
+
+template <typename R, int VEC>
+__global__ __launch_bounds__(kBlock) void feature_forward_kernel(const Args<R> a) {
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int slices = C / VEC;
+  const int64_t total = a.voxels() * N * slices;
+  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * kBlock) {
+    const int64_t row = e / slices;  // (voxel, view)
+    const int c0 = (int)(e - row * slices) * VEC;
+    const int64_t i = row / N;
+    const int n = (int)(row - i * N);
+    const Voxel<R> v = locate(a, i);
+    Sample<R> s;
+    const int64_t cam = (int64_t)v.b * N + n;
+    project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+    Slice<R, VEC> out;
+    if (s.state == 2) {
+      const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
+      const Slice<R, VEC> v00 = load_slice<R, VEC>(t.t00 + c0), v01 = load_slice<R, VEC>(t.t01 + c0),
+                          v11 = load_slice<R, VEC>(t.t11 + c0), v10 = load_slice<R, VEC>(t.t10 + c0);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        out.v[k] = s.k00 * v00.v[k] + s.k01 * v01.v[k] + s.k11 * v11.v[k] + s.k10 * v10.v[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) out.v[k] = R(0);
+    }
+    store_slice<R, VEC>(a.cost + row * C + c0, out);
+    if (c0 == 0) a.mask[row] = s.state == 2 ? 1 : 0;
+  }
+}
+
+template <typename R, int VEC>
+__global__ __launch_bounds__(kBlock) void feature_backward_kernel(const Args<R> a) {
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int slices = C / VEC;
+  const int64_t total = a.voxels() * N * slices;
+  const int64_t row_step = (int64_t)srcW * C;
+  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * kBlock) {
+    const int64_t row = e / slices;
+    const int c0 = (int)(e - row * slices) * VEC;
+    if (a.mask_in[row] == 0) continue;  // :261-263
+    const int64_t i = row / N;
+    const int n = (int)(row - i * N);
+    const Voxel<R> v = locate(a, i);
+    Sample<R> s;
+    const int64_t cam = (int64_t)v.b * N + n;
+    project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+    // the reference trusts the mask (:271, :284-285); a sample that is not accepted any more
+    // is skipped instead of read out of bounds
+    if (s.state != 2) continue;
+    const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
+    R *g00 = a.src_grad + (t.t00 - a.src) + c0;
+    const Slice<R, VEC> g = load_slice<R, VEC>(a.cost_grad + row * C + c0);
+    const Slice<R, VEC> v00 = load_slice<R, VEC>(t.t00 + c0), v01 = load_slice<R, VEC>(t.t01 + c0),
+                        v11 = load_slice<R, VEC>(t.t11 + c0), v10 = load_slice<R, VEC>(t.t10 + c0);
+    R h_grad = R(0), w_grad = R(0);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      atomic_add(g00 + k, g.v[k] * s.k00);
+      atomic_add(g00 + C + k, g.v[k] * s.k01);
+      atomic_add(g00 + C + row_step + k, g.v[k] * s.k11);
+      atomic_add(g00 + row_step + k, g.v[k] * s.k10);
+      const R t1 = v11.v[k] - v10.v[k] - v01.v[k] + v00.v[k];
+      h_grad += g.v[k] * (t1 * s.dw + v10.v[k] - v00.v[k]);
+      w_grad += g.v[k] * (t1 * s.dh + v01.v[k] - v00.v[k]);
+    }
+    atomic_add(a.depth_grad + v.pix, depth_chain(s, h_grad, w_grad));
+  }
+}
+
+template <typename R>
+bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+}  // namespace
+
+template <typename S>
+hipError_t launch_v3_forward(const Args<S> &a, hipStream_t stream) {
+  const int64_t total = a.voxels();
+  if (total == 0) return hipSuccess;
+  const int grid = grid_for(total, kBlock);
+  if (a.reduce == 0)
+    v3_forward_kernel<S, 0><<<grid, kBlock, 0, stream>>>(a);
+  else
+    v3_forward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  return hipGetLastError();
+}
+
+template <typename S>
+hipError_t launch_v3_backward(const Args<S> &a, hipStream_t stream) {
+  hipError_t err;
+  if ((err = launch_fill_zero(a.ref_grad, (size_t)(a.pixels() * a.C) * sizeof(S), stream)) != hipSuccess)
+    return err;
+  if ((err = launch_fill_zero(a.src_grad, (size_t)(a.B * a.N * a.srcH * a.srcW * a.C) * sizeof(S),
+                              stream)) != hipSuccess)
+    return err;
+  if ((err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(S), stream)) != hipSuccess)
+    return err;
+  const int64_t total = a.voxels();
+  if (total == 0 || a.C == 0) return hipSuccess;
+  const int grid = grid_for(total, kBlock);
+  if (a.reduce == 0)
+    v3_backward_kernel<S, 0><<<grid, kBlock, 0, stream>>>(a);
+  else
+    v3_backward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  return hipGetLastError();
+}
+
+template <typename S>
+hipError_t launch_feature_forward(const Args<S> &a, hipStream_t stream) {
+  constexpr int kVec = 16 / (int)sizeof(S);
+  const bool wide = a.C % kVec == 0 && aligned16<S>(a.src) && aligned16<S>(a.cost);
+  const int64_t total = a.voxels() * a.N * (wide ? a.C / kVec : a.C);
+  if (total == 0) return hipSuccess;
+  const int grid = grid_for(total, kBlock);
+  if (wide)
+    feature_forward_kernel<S, kVec><<<grid, kBlock, 0, stream>>>(a);
+  else
+    feature_forward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  return hipGetLastError();
+}
+
+template <typename S>
+hipError_t launch_feature_backward(const Args<S> &a, hipStream_t stream) {
+  hipError_t err;
+  if ((err = launch_fill_zero(a.src_grad, (size_t)(a.B * a.N * a.srcH * a.srcW * a.C) * sizeof(S),
+                              stream)) != hipSuccess)
+    return err;
+  if ((err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(S), stream)) != hipSuccess)
+    return err;
+  constexpr int kVec = 16 / (int)sizeof(S);
+  const bool wide = a.C % kVec == 0 && aligned16<S>(a.src) && aligned16<S>(a.cost_grad);
+  const int64_t total = a.voxels() * a.N * (wide ? a.C / kVec : a.C);
+  if (total == 0) return hipSuccess;
+  const int grid = grid_for(total, kBlock);
+  if (wide)
+    feature_backward_kernel<S, kVec><<<grid, kBlock, 0, stream>>>(a);
+  else
+    feature_backward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  return hipGetLastError();
+}
+
+#define CHOP_INSTANTIATE(S)                                                       \
+  template hipError_t launch_v3_forward<S>(const Args<S> &, hipStream_t);         \
+  template hipError_t launch_v3_backward<S>(const Args<S> &, hipStream_t);        \
+  template hipError_t launch_feature_forward<S>(const Args<S> &, hipStream_t);    \
+  template hipError_t launch_feature_backward<S>(const Args<S> &, hipStream_t);
+CHOP_INSTANTIATE(float)
+CHOP_INSTANTIATE(double)
+#undef CHOP_INSTANTIATE
+
+}  // namespace chop

@@ -1,8 +1,9 @@
 """Host-side mirror of the reference's Python operator interface for the cost volume.
 
 Same names, argument order, defaults and outputs as
-custom_helper_op/python/ops/custom_helper_ops.py:32-96 and :133-163 (``cost_volume``,
-``cost_volume_v2``, ``cost_aggregate`` and the gradients registered for them), with torch tensors standing in
+custom_helper_op/python/ops/custom_helper_ops.py:32-197 (``cost_volume``,
+``cost_volume_v2``, ``cost_volume_v3``, ``cost_aggregate``, ``feature_aggregate`` and the
+gradients registered for them), with torch tensors standing in
 for TensorFlow tensors: torch supplies device memory and the current HIP stream, the
 arithmetic is done by ``libchop_costvol.so`` through its C ABI.  The shape checks are the
 ones ``CostVolumeOp::Compute`` performs (custom_helper_op/cc/kernels/
@@ -285,6 +286,140 @@ def cost_aggregate_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost
     return ref_grad, src_grad, bp_grad
 
 
+def _check_v3_groups(C, groups):
+    # cost_volume_kernels_v3.cc:111-115
+    _require(isinstance(groups, int) and groups > 0 and C % groups == 0,
+             "image_channels and groups_ must match")
+    _require(C // groups <= 8, "image_channels / groups_ less than MAX_SUBCHANNELS_SIZE(8)")
+
+
+def cost_volume_v3_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
+                       groups=None, half_centor=True):
+    """The ``CostVolumeV3`` op without autograd: ``(cost [B,H,W,D,1], cost_mask int32
+    [B,H,W,D,1] (MEAN) or [B,H,W,D,3] (MIN: view, reference group, source group))``
+    (shapes: custom_helper_op/cc/ops/custom_helper_ops.cc:311-347; checks:
+    cost_volume_kernels_v3.cc:94-115).  float32 and float64, as registered."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, dt, dev, "base_plane")
+    offsets = _prep(offsets, dt, dev, "offsets")
+    Rs, Ts = _prep(Rs, dt, dev, "Rs"), _prep(Ts, dt, dev, "Ts")
+    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, Rs, Ts)
+    _check_v3_groups(C, groups)
+    cost = torch.empty((B, H, W, D, 1), dtype=dt, device=dev)
+    mask = torch.empty((B, H, W, D, 1 if red == 0 else 3), dtype=torch.int32, device=dev)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    fn = lib.chop_cost_volume_v3_fwd_f32 if dt == torch.float32 else lib.chop_cost_volume_v3_fwd_f64
+    rc = fn(_stream(cost), red, int(half_centor), *dims, groups, _ptr(ref_image), _ptr(src_images),
+            _ptr(base_plane), _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(cost), _ptr(mask))
+    _lib.check(rc)
+    return cost, mask
+
+
+def cost_volume_grad_v3(ref_image, src_images, base_plane, offsets, rs, ts, cost_grad, cost_mask,
+                        reduce_method="MEAN", groups=None, half_centor=True):
+    """The ``CostVolumeGradV3`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``
+    (checks: cost_volume_kernels_v3.cc:231-255)."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    dt, dev = ref_image.dtype, ref_image.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    ref_image = _prep(ref_image, dt, dev, "ref_image")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, dt, dev, "base_plane")
+    offsets = _prep(offsets, dt, dev, "offsets")
+    rs, ts = _prep(rs, dt, dev, "Rs"), _prep(ts, dt, dev, "Ts")
+    cost_grad = _prep(cost_grad, dt, dev, "cost_grad")
+    cost_mask = _prep(cost_mask, torch.int32, dev, "cost_mask")
+    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, rs, ts)
+    _check_v3_groups(C, groups)
+    _require(tuple(cost_grad.shape) == (B, H, W, D, 1),
+             "cost_grad must have rank 5, and must compate to ref_image")
+    _require(tuple(cost_mask.shape) == (B, H, W, D, 1 if red == 0 else 3),
+             "cost_mask must have rank 5, and must compate to ref_image")
+    ref_grad = torch.empty_like(ref_image)
+    src_grad = torch.empty_like(src_images)
+    bp_grad = torch.empty_like(base_plane)
+    dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
+    fn = lib.chop_cost_volume_v3_bwd_f32 if dt == torch.float32 else lib.chop_cost_volume_v3_bwd_f64
+    rc = fn(_stream(ref_grad), red, int(half_centor), *dims, groups, _ptr(ref_image),
+            _ptr(src_images), _ptr(base_plane), _ptr(offsets), _ptr(rs), _ptr(ts), _ptr(cost_grad),
+            _ptr(cost_mask), _ptr(ref_grad), _ptr(src_grad), _ptr(bp_grad))
+    _lib.check(rc)
+    return ref_grad, src_grad, bp_grad
+
+
+def _check_feature(src_images, base_plane, offsets, Rs, Ts):
+    # feature_aggregate_kernels.cc:69-92
+    _require(src_images.dim() == 5, "src_images must have rank 5")
+    B, N, srcH, srcW, C = src_images.shape
+    _require(base_plane.dim() == 4 and base_plane.shape[0] == B and base_plane.shape[3] == 1,
+             "base_plane must have rank 4, and must compate to ref_image")
+    H, W = base_plane.shape[1:3]
+    _require(offsets.dim() == 2 and offsets.shape[0] == B,
+             "offsets must have rank 2, and must compate to ref_image")
+    _require(Rs.dim() == 4 and tuple(Rs.shape) == (B, N, 3, 3),
+             "Rs must have rank 2, and must compate to ref_image")
+    _require(Ts.dim() == 3 and tuple(Ts.shape) == (B, N, 3),
+             "Ts must have rank 2, and must compate to ref_image")
+    return B, H, W, C, offsets.shape[1], N, srcH, srcW
+
+
+def feature_aggregate_raw(src_images, base_plane, offsets, Rs, Ts, half_centor=True):
+    """The ``FeatureAggregate`` op without autograd: ``(mapped_feature [B,H,W,D,N,C],
+    mapped_mask int32 [B,H,W,D,N,1])``; H and W are base_plane's (shapes:
+    custom_helper_op/cc/ops/custom_helper_ops.cc:414-440)."""
+    lib = _lib.load()
+    dt, dev = src_images.dtype, src_images.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, dt, dev, "base_plane")
+    offsets = _prep(offsets, dt, dev, "offsets")
+    Rs, Ts = _prep(Rs, dt, dev, "Rs"), _prep(Ts, dt, dev, "Ts")
+    B, H, W, C, D, N, srcH, srcW = dims = _check_feature(src_images, base_plane, offsets, Rs, Ts)
+    mapped = torch.empty((B, H, W, D, N, C), dtype=dt, device=dev)
+    mask = torch.empty((B, H, W, D, N, 1), dtype=torch.int32, device=dev)
+    fn = (lib.chop_feature_aggregate_fwd_f32 if dt == torch.float32
+          else lib.chop_feature_aggregate_fwd_f64)
+    rc = fn(_stream(mapped), int(half_centor), *dims, _ptr(src_images), _ptr(base_plane),
+            _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(mapped), _ptr(mask))
+    _lib.check(rc)
+    return mapped, mask
+
+
+def feature_aggregate_grad(src_images, base_plane, offsets, rs, ts, mapped_feature_grad,
+                           mapped_mask, half_centor=True):
+    """The ``FeatureAggregateGrad`` op: ``(src_images_grad, base_plane_grad)``
+    (checks: feature_aggregate_kernels.cc:176-210)."""
+    lib = _lib.load()
+    dt, dev = src_images.dtype, src_images.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    src_images = _prep(src_images, dt, dev, "src_images")
+    base_plane = _prep(base_plane, dt, dev, "base_plane")
+    offsets = _prep(offsets, dt, dev, "offsets")
+    rs, ts = _prep(rs, dt, dev, "Rs"), _prep(ts, dt, dev, "Ts")
+    mapped_feature_grad = _prep(mapped_feature_grad, dt, dev, "mapped_feature_grad")
+    mapped_mask = _prep(mapped_mask, torch.int32, dev, "mapped_mask")
+    B, H, W, C, D, N, srcH, srcW = dims = _check_feature(src_images, base_plane, offsets, rs, ts)
+    _require(tuple(mapped_feature_grad.shape) == (B, H, W, D, N, C),
+             "mapped_feature_grad must have rank 6, and must compate to src_images")
+    _require(tuple(mapped_mask.shape) == (B, H, W, D, N, 1),
+             "mapped_mask must have rank 6, and must compate to src_images")
+    src_grad = torch.empty_like(src_images)
+    bp_grad = torch.empty_like(base_plane)
+    fn = (lib.chop_feature_aggregate_bwd_f32 if dt == torch.float32
+          else lib.chop_feature_aggregate_bwd_f64)
+    rc = fn(_stream(src_grad), int(half_centor), *dims, _ptr(src_images), _ptr(base_plane),
+            _ptr(offsets), _ptr(rs), _ptr(ts), _ptr(mapped_feature_grad), _ptr(mapped_mask),
+            _ptr(src_grad), _ptr(bp_grad))
+    _lib.check(rc)
+    return src_grad, bp_grad
+
+
 class _CostVolume(torch.autograd.Function):
     """Forward = CostVolume, backward = the gradient registered for it
     (custom_helper_ops.py:41-61): the Grad op is fed the forward's cost_mask, the incoming
@@ -347,6 +482,46 @@ class _CostAggregate(torch.autograd.Function):
         return rg, sg, bg, None, None, None, None, None
 
 
+class _CostVolumeV3(torch.autograd.Function):
+    """CostVolumeV3 with its registered gradient (custom_helper_ops.py:107-131)."""
+
+    @staticmethod
+    def forward(ctx, ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method, groups,
+                half_centor):
+        cost, mask = cost_volume_v3_raw(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                        reduce_method, groups, half_centor)
+        ctx.save_for_backward(ref_image, src_images, base_plane, offsets, Rs, Ts, mask)
+        ctx.attrs = (reduce_method, groups, half_centor)
+        ctx.mark_non_differentiable(mask)
+        return cost, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        ref_image, src_images, base_plane, offsets, Rs, Ts, mask = ctx.saved_tensors
+        rg, sg, bg = cost_volume_grad_v3(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                         grad_out.contiguous(), mask, *ctx.attrs)
+        return rg, sg, bg, None, None, None, None, None, None
+
+
+class _FeatureAggregate(torch.autograd.Function):
+    """FeatureAggregate with its registered gradient (custom_helper_ops.py:174-195)."""
+
+    @staticmethod
+    def forward(ctx, src_images, base_plane, offsets, Rs, Ts, half_centor):
+        mapped, mask = feature_aggregate_raw(src_images, base_plane, offsets, Rs, Ts, half_centor)
+        ctx.save_for_backward(src_images, base_plane, offsets, Rs, Ts, mask)
+        ctx.half_centor = half_centor
+        ctx.mark_non_differentiable(mask)
+        return mapped, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        src_images, base_plane, offsets, Rs, Ts, mask = ctx.saved_tensors
+        sg, bg = feature_aggregate_grad(src_images, base_plane, offsets, Rs, Ts,
+                                        grad_out.contiguous(), mask, ctx.half_centor)
+        return sg, bg, None, None, None, None
+
+
 def cost_volume(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
                 half_centor=True, name=None):
     """``custom_helper_op.cost_volume``: returns ``(cost, cost_mask)``; differentiable with
@@ -381,6 +556,30 @@ def cost_aggregate(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_me
     Ts = torch.as_tensor(Ts, device=ref_image.device)
     return _CostAggregate.apply(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method,
                                 half_centor)
+
+
+def cost_volume_v3(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
+                   groups=None, half_centor=True, name=None):
+    """``custom_helper_op.cost_volume_v3`` (custom_helper_ops.py:99-104): returns
+    ``(cost [B,H,W,D,1], cost_mask)``; differentiable with respect to ref_image, src_images and
+    base_plane."""
+    del name
+    offsets = torch.as_tensor(offsets, device=ref_image.device)
+    Rs = torch.as_tensor(Rs, device=ref_image.device)
+    Ts = torch.as_tensor(Ts, device=ref_image.device)
+    return _CostVolumeV3.apply(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method,
+                               groups, half_centor)
+
+
+def feature_aggregate(src_images, base_plane, offsets, Rs, Ts, half_centor=True, name=None):
+    """``custom_helper_op.feature_aggregate`` (custom_helper_ops.py:166-171): returns
+    ``(mapped_feature [B,H,W,D,N,C], mapped_mask [B,H,W,D,N,1])``; differentiable with respect
+    to src_images and base_plane."""
+    del name
+    offsets = torch.as_tensor(offsets, device=src_images.device)
+    Rs = torch.as_tensor(Rs, device=src_images.device)
+    Ts = torch.as_tensor(Ts, device=src_images.device)
+    return _FeatureAggregate.apply(src_images, base_plane, offsets, Rs, Ts, half_centor)
 
 
 def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):

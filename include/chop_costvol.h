@@ -155,6 +155,87 @@ int chop_cost_aggregate_bwd_f64(void *stream, int reduce, int half_centor, int64
                                 const int32_t *mask, double *ref_grad, double *src_grad,
                                 double *base_plane_grad);
 
+/* ---- CostVolumeV3 forward / backward -------------------------------------------------
+ * Per accepted view, the largest dot product between any channel group of the bilinear
+ * source sample and any channel group of the reference pixel (groups x groups pairs of
+ * C/groups channels each, at most 8 channels per group); one value per voxel.
+ * Replaces functor::CostVolumeV3Functor<GPUDevice,T,half_centor>::operator() and
+ * functor::CostVolumeGradV3Functor<GPUDevice,T,half_centor>::operator()
+ * (declared custom_helper_op/cc/kernels/cost_volume_v3.h:40-141, defined
+ * cost_volume_kernels_gpu_v3.cu.cc:323-369 and :653-719, called from
+ * CostVolumeV3Op::Compute and CostVolumeGradV3Op::Compute,
+ * cost_volume_kernels_v3.cc:137-145 and :274-282).
+ * cost is [B,H,W,D,1].  MEAN: mask int32 [B,H,W,D,1] = number of accepted views, cost =
+ * mean of the views' maxima (each seeded with the smallest positive normal number, as the
+ * reference does), 0 where no view was accepted.  MIN: cost = the largest value over all
+ * views and pairs, mask int32 [B,H,W,D,3] = (view, reference group, source group) of the
+ * winner, all -1 and cost 0 when nothing exceeded the seed.
+ * The backward takes cost_grad [B,H,W,D,1] and the forward's mask.  A view whose best
+ * pair does not exceed the seed contributes no gradient (the reference indexes channel
+ * group -1 there, cost_volume_kernels_gpu_v3.cu.cc:495-496).
+ * Extra status: CHOP_ERR_BAD_GROUPS when groups does not divide C or C/groups > 8
+ * (cost_volume_kernels_v3.cc:111-115). */
+int chop_cost_volume_v3_fwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const float *ref, const float *src,
+                                const float *base_plane, const float *offsets, const float *Rs,
+                                const float *Ts, float *cost, int32_t *mask);
+int chop_cost_volume_v3_fwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const double *ref, const double *src,
+                                const double *base_plane, const double *offsets,
+                                const double *Rs, const double *Ts, double *cost, int32_t *mask);
+int chop_cost_volume_v3_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const float *ref, const float *src,
+                                const float *base_plane, const float *offsets, const float *Rs,
+                                const float *Ts, const float *cost_grad, const int32_t *mask,
+                                float *ref_grad, float *src_grad, float *base_plane_grad);
+int chop_cost_volume_v3_bwd_f64(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
+                                int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
+                                int64_t srcW, int groups, const double *ref, const double *src,
+                                const double *base_plane, const double *offsets,
+                                const double *Rs, const double *Ts, const double *cost_grad,
+                                const int32_t *mask, double *ref_grad, double *src_grad,
+                                double *base_plane_grad);
+
+/* ---- FeatureAggregate forward / backward ---------------------------------------------
+ * The warp alone: mapped_feature [B,H,W,D,N,C] holds the bilinear sample of every source
+ * view at every voxel (zeros where the view is not accepted) and mapped_mask int32
+ * [B,H,W,D,N,1] is 1 / 0.  H and W are those of base_plane [B,H,W,1]; the source images
+ * [B,N,srcH,srcW,C] may have another size.
+ * Replaces functor::FeatureAggregateFunctor<GPUDevice,T,half_centor>::operator() and
+ * functor::FeatureAggregateGradFunctor<GPUDevice,T,half_centor>::operator()
+ * (declared custom_helper_op/cc/kernels/feature_aggregate.h:36-128, defined
+ * feature_aggregate_kernels_gpu.cu.cc:182-213 and :339-388, called from
+ * FeatureAggregateOp::Compute and FeatureAggregateGradOp::Compute,
+ * feature_aggregate_kernels.cc:105-113 and :223-231).
+ * The backward takes mapped_feature_grad [B,H,W,D,N,C] and the forward's mask and writes
+ * src_grad [B,N,srcH,srcW,C] and base_plane_grad [B,H,W,1]. */
+int chop_feature_aggregate_fwd_f32(void *stream, int half_centor, int64_t B, int64_t H, int64_t W,
+                                   int64_t C, int64_t D, int64_t N, int64_t srcH, int64_t srcW,
+                                   const float *src, const float *base_plane,
+                                   const float *offsets, const float *Rs, const float *Ts,
+                                   float *mapped_feature, int32_t *mapped_mask);
+int chop_feature_aggregate_fwd_f64(void *stream, int half_centor, int64_t B, int64_t H, int64_t W,
+                                   int64_t C, int64_t D, int64_t N, int64_t srcH, int64_t srcW,
+                                   const double *src, const double *base_plane,
+                                   const double *offsets, const double *Rs, const double *Ts,
+                                   double *mapped_feature, int32_t *mapped_mask);
+int chop_feature_aggregate_bwd_f32(void *stream, int half_centor, int64_t B, int64_t H, int64_t W,
+                                   int64_t C, int64_t D, int64_t N, int64_t srcH, int64_t srcW,
+                                   const float *src, const float *base_plane,
+                                   const float *offsets, const float *Rs, const float *Ts,
+                                   const float *mapped_feature_grad, const int32_t *mapped_mask,
+                                   float *src_grad, float *base_plane_grad);
+int chop_feature_aggregate_bwd_f64(void *stream, int half_centor, int64_t B, int64_t H, int64_t W,
+                                   int64_t C, int64_t D, int64_t N, int64_t srcH, int64_t srcW,
+                                   const double *src, const double *base_plane,
+                                   const double *offsets, const double *Rs, const double *Ts,
+                                   const double *mapped_feature_grad,
+                                   const int32_t *mapped_mask, double *src_grad,
+                                   double *base_plane_grad);
+
 /* ---- 16-bit storage extension --------------------------------------------------------
  * No counterpart in the reference, whose ops register float32 and float64 only
  * (custom_helper_ops.cc:197,234).  ref, src, cost, cost_grad, ref_grad and src_grad

@@ -183,6 +183,83 @@ def cost_volume_v2_bwd(ref, src, depth_grid, Rs, Ts, cost_grad, mask, reduce="ME
     return ref_grad, src_grad, dg_grad
 
 
+def cost_volume_v3_fwd(ref, src, base_plane, offsets, Rs, Ts, reduce="MEAN", groups=1,
+                       half_centor=True, threads=1):
+    """cost [B,H,W,D,1]; mask [B,H,W,D,1] (MEAN) or [B,H,W,D,3] (MIN: view, ref group, src group)."""
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, base_plane, offsets, Rs, Ts = (_c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts))
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = offsets.shape[1]
+    r = _REDUCE[reduce]
+    cost = np.empty((B, H, W, D, 1), dt)
+    mask = np.empty((B, H, W, D, 1 if r == 0 else 3), np.int32)
+    fn = getattr(lib(), "chop_oracle_cost_volume_v3_fwd_" + sfx)
+    rc = fn(r, int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW, int(groups)), _p(ref),
+            _p(src), _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
+    _check(rc, "cost_volume_v3_fwd")
+    return cost, mask
+
+
+def cost_volume_v3_bwd(ref, src, base_plane, offsets, Rs, Ts, cost_grad, mask, reduce="MEAN",
+                       groups=1, half_centor=True, threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, base_plane, offsets, Rs, Ts, cost_grad = (
+        _c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts, cost_grad))
+    mask = _c(mask, np.int32)
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = offsets.shape[1]
+    ref_grad = np.empty_like(ref)
+    src_grad = np.empty_like(src)
+    bp_grad = np.empty_like(base_plane)
+    fn = getattr(lib(), "chop_oracle_cost_volume_v3_bwd_" + sfx)
+    rc = fn(_REDUCE[reduce], int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW, int(groups)),
+            _p(ref), _p(src), _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost_grad),
+            _p(mask), _p(ref_grad), _p(src_grad), _p(bp_grad), int(threads))
+    _check(rc, "cost_volume_v3_bwd")
+    return ref_grad, src_grad, bp_grad
+
+
+def feature_aggregate_fwd(src, base_plane, offsets, Rs, Ts, half_centor=True, threads=1):
+    """mapped_feature [B,H,W,D,N,C] and mapped_mask [B,H,W,D,N,1]; H, W from base_plane."""
+    dt = src.dtype
+    sfx = _sfx(dt)
+    src, base_plane, offsets, Rs, Ts = (_c(x, dt) for x in (src, base_plane, offsets, Rs, Ts))
+    B, N, sH, sW, C = src.shape
+    H, W = base_plane.shape[1:3]
+    D = offsets.shape[1]
+    mapped = np.empty((B, H, W, D, N, C), dt)
+    mask = np.empty((B, H, W, D, N, 1), np.int32)
+    fn = getattr(lib(), "chop_oracle_feature_aggregate_fwd_" + sfx)
+    rc = fn(int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(src), _p(base_plane),
+            _p(offsets), _p(Rs), _p(Ts), _p(mapped), _p(mask), int(threads))
+    _check(rc, "feature_aggregate_fwd")
+    return mapped, mask
+
+
+def feature_aggregate_bwd(src, base_plane, offsets, Rs, Ts, mapped_grad, mapped_mask,
+                          half_centor=True, threads=1):
+    dt = src.dtype
+    sfx = _sfx(dt)
+    src, base_plane, offsets, Rs, Ts, mapped_grad = (
+        _c(x, dt) for x in (src, base_plane, offsets, Rs, Ts, mapped_grad))
+    mapped_mask = _c(mapped_mask, np.int32)
+    B, N, sH, sW, C = src.shape
+    H, W = base_plane.shape[1:3]
+    D = offsets.shape[1]
+    src_grad = np.empty_like(src)
+    bp_grad = np.empty_like(base_plane)
+    fn = getattr(lib(), "chop_oracle_feature_aggregate_bwd_" + sfx)
+    rc = fn(int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(src), _p(base_plane),
+            _p(offsets), _p(Rs), _p(Ts), _p(mapped_grad), _p(mapped_mask), _p(src_grad),
+            _p(bp_grad), int(threads))
+    _check(rc, "feature_aggregate_bwd")
+    return src_grad, bp_grad
+
+
 def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):
     """Per-(voxel, view) source coordinates ``[B,H,W,D,N]``: (sw, sh, fh, fw, state)."""
     if depth_grid is not None:
