@@ -258,6 +258,13 @@ int feature_call(void *stream, int half_centor, const Dims &d, const S *src, con
   a.cost = mapped, a.mask = mapped_mask, a.cost_grad = mapped_grad, a.mask_in = mask_in;
   a.src_grad = src_grad, a.depth_grad = base_plane_grad;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (g_kernel_family == 0 && work) {
+    if (backward ? tiled_backward_supported(a) : tiled_forward_supported(a)) {
+      g_last_family = 2;
+      return backward ? launch_status(launch_tiled_backward(a, s), "tiled FeatureAggregate backward launch")
+                      : launch_status(launch_tiled_forward(a, s), "tiled FeatureAggregate forward launch");
+    }
+  }
   g_last_family = 1;
   if (backward) return launch_status(launch_feature_backward(a, s), "FeatureAggregate backward launch");
   return launch_status(launch_feature_forward(a, s), "FeatureAggregate forward launch");

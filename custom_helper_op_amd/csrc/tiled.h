@@ -397,7 +397,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
                       static_cast<float>(t.h) + half, cam);
   const float base = a.depth_grid ? 0.f : a.base_plane[t.pix];
   float ref[VEC];
-  load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+  if constexpr (CORR != 4) {
+    load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+  } else {
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) ref[c] = 0.f;  // the warp-only op has no reference image
+  }
   const S *view[NV];
 #pragma unroll
   for (int n = 0; n < NV; ++n)
@@ -410,7 +415,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
   for (int n = 0; n < NV; ++n) cur[n] = -1;
 
   // CORR: 0 squared difference per channel, 1 group correlation, 2 squared difference
-  // summed over all channels (one value per voxel)
+  // summed over all channels (one value per voxel), 4 the samples themselves, one row per
+  // (voxel, view), and a 0/1 mask per (voxel, view)
+  // (feature_aggregate_kernels_gpu.cu.cc:33-121)
   const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
   const int gv = VEC / g.sub;  // output values per lane
   const int d_lo = t.d_lo, d_hi = t.d_hi;
@@ -430,6 +437,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
         if (n < N && d_ok) reproject<NV>(cam, n, depth, half, g.src_h_max, g.src_w_max, srcW, C, hit);
         cnt += hit.off >= 0;
+        if constexpr (CORR == 4) {
+          if (n < N && d_ok && t.pix_ok)
+            __builtin_nontemporal_store(hit.off >= 0 ? 1 : 0, a.mask + (t.pix * D + d) * N + n);
+        }
         if constexpr (LPP > 1) {
           lds_at<int>(smem, q4, kOff + (n * LPP * PPW) * 4) = hit.off;
           lds_at<float4>(smem, q4 * 4u, kWts + (n * LPP * PPW) * 16) =
@@ -439,7 +450,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           r_wts[n] = make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
         }
       }
-      if constexpr (REDUCE == 0)
+      if constexpr (REDUCE == 0 && CORR != 4)
         if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
     }
     if constexpr (LPP > 1) wave_sync();
@@ -448,7 +459,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
-      if (d >= d_hi) break;
+      if (d >= d_hi) {
+        // (a `break` gives the widest tile a run-time trip count, which keeps the compiler
+        // from unrolling it and sends its register arrays to scratch memory)
+        if constexpr (LPP >= 16) continue; else break;
+      }
       float acc[VEC];
       int arg[VEC];  // REDUCE == 1: winning view per channel (or per group)
 #pragma unroll
@@ -469,6 +484,30 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         } else {
           off = r_off[n];
           wt = r_wts[n];
+        }
+        if constexpr (CORR == 4) {
+          // the sample in the reference's operand order (bit-identical to the plain
+          // evaluation), zeros for a view that is not accepted
+          float smp[VEC];
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) smp[c] = 0.f;
+          if (off >= 0) {
+            if (off != cur[n]) {
+              cur[n] = off;
+              const S *q = view[n] + off;
+              load_vec<S, VEC, false>(q, tap[n][0]);
+              load_vec<S, VEC, false>(q + C, tap[n][1]);
+              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
+              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
+            }
+#pragma unroll
+            for (int c = 0; c < VEC; ++c)
+              smp[c] = wt.x * tap[n][0][c] + wt.y * tap[n][1][c] + wt.z * tap[n][2][c] +
+                       wt.w * tap[n][3][c];
+          }
+          if (n < N && t.pix_ok)
+            store_vec<S, VEC, true>(a.cost + ((t.pix * D + d) * N + n) * C + t.cl * VEC, smp);
+          continue;
         }
         if (off >= 0) {
           if (off != cur[n]) {
@@ -532,6 +571,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
           ++k;
         }
       }
+      if constexpr (CORR == 4) continue;  // every view's row is already stored
       if constexpr (REDUCE == 1) {
         if (t.pix_ok) {
           S *out = a.cost + (t.pix * D + d) * OC;
@@ -807,7 +847,13 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
                       static_cast<float>(t.h) + half, cam);
   const float base = per_voxel_depth ? 0.f : a.base_plane[t.pix];
   float ref[VEC];
-  load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+  if constexpr (CORR != 4) {
+    load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+  } else {
+    static_assert(CORR != 4 || NV == 1, "the warp-only gradient runs one view per workgroup");
+#pragma unroll
+    for (int c = 0; c < VEC; ++c) ref[c] = 0.f;
+  }
   const int64_t view_elems = (int64_t)srcH * srcW * C;
   float *src_grad_img = kWide ? a.src_grad_acc : reinterpret_cast<float *>(a.src_grad);
   const S *view[NV];
@@ -842,7 +888,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   wave_sync();
 
   // CORR: 0 squared difference per channel, 1 group correlation, 2 squared difference
-  // summed over all channels (one upstream gradient per voxel)
+  // summed over all channels (one upstream gradient per voxel), 4 the warp alone: one
+  // upstream-gradient row and one 0/1 mask entry per (voxel, view)
+  // (feature_aggregate_kernels_gpu.cu.cc:219-326)
   const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
@@ -850,9 +898,15 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   constexpr int PFMAX = REDUCE ? 4 : 8;
   constexpr int PF = LPP < PFMAX ? LPP : PFMAX;
   constexpr bool kMaskRows = REDUCE == 1 && CORR != 2;
-  const S *cg_lane = a.cost_grad + t.pix * D * OC + (CORR == 2 ? 0 : t.cl * (CORR ? gv : VEC));
+  // element steps from one depth to the next in the upstream gradient and in the mask
+  const int cg_step = CORR == 4 ? N * C : OC;
+  const int cnt_step = kMaskRows ? OC : CORR == 4 ? N : 1;
+  const S *cg_lane =
+      CORR == 4 ? a.cost_grad + (t.pix * D * N + t.view0) * C + t.cl * VEC
+                : a.cost_grad + t.pix * D * OC + (CORR == 2 ? 0 : t.cl * (CORR ? gv : VEC));
   const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
-  const int32_t *cnt_src = a.mask_in + t.pix * D * (kMaskRows ? OC : 1);
+  const int32_t *cnt_src = CORR == 4 ? a.mask_in + t.pix * D * N + t.view0
+                                     : a.mask_in + t.pix * D * (kMaskRows ? OC : 1);
   const int32_t *mask_lane = cnt_src + t.cl * (CORR ? gv : VEC);  // this lane's part of a mask row
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
     // Depth hypothesis and valid-view count of lane (p, j)'s voxel: requested before the
@@ -862,7 +916,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     int cnt = REDUCE ? -1 : 0;  // "nothing to do" for a lane without a voxel
     if (d0 + t.cl < d_hi) {
       dv = dv_src[d0 + t.cl];
-      if (t.pix_ok) cnt = cnt_src[(int64_t)(d0 + t.cl) * (kMaskRows ? OC : 1)];
+      if (t.pix_ok) cnt = cnt_src[(int64_t)(d0 + t.cl) * cnt_step];
       if constexpr (CORR == 2)  // the voxel's one upstream gradient rides with its record
         cg_vox = reinterpret_cast<const float *>(cg_lane)[d0 + t.cl];
     }
@@ -880,8 +934,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
       for (int jj = 0; jj < PF; ++jj) {
         const int d = min(first + jj, d_hi - 1);
-        const S *src_cg = cg_lane + (int64_t)d * OC;
-        if (CORR == 0)
+        const S *src_cg = cg_lane + (int64_t)d * cg_step;
+        if (CORR == 0 || CORR == 4)
           load_vec<S, VEC, true>(src_cg, cgr[jj]);
         else
           load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
@@ -1012,7 +1066,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
-      if (d >= d_hi) break;
+      if (d >= d_hi) {
+        if constexpr (LPP >= 16) continue; else break;  // see the forward kernel
+      }
       if constexpr (LPP > PF && CORR != 2) {
         if (jj > 0 && jj % PF == 0) load_rows(d0 + jj);  // next part of a deep chunk
       }
@@ -1098,7 +1154,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
               float gsrc;  // d(loss)/d(sample of this channel)
-              if (CORR != 1) {
+              if constexpr (CORR == 4) {
+                gsrc = cg[c];
+              } else if (CORR != 1) {
                 float diff = __builtin_fmaf(wt.x, tap[n][0][c], -ref[c]);
                 diff = __builtin_fmaf(wt.y, tap[n][1][c], diff);
                 diff = __builtin_fmaf(wt.z, tap[n][2][c], diff);
@@ -1173,7 +1231,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   // atomic add per depth segment into the zero-filled outputs
   float *rg = kWide ? a.ref_grad_acc : reinterpret_cast<float *>(a.ref_grad);
   const bool single = g.nseg * g.ngroups == 1;
-  if (single) {
+  if constexpr (CORR == 4) {
+    // no reference image, no gradient for it
+  } else if (single) {
     if (t.pix_ok) {
       if (kWide)
         store_vec<float, VEC, false>(rg + t.pix * C + t.cl * VEC, racc);

@@ -175,6 +175,33 @@ def test_feature_backward(oracle, shape, dtype):
             assert_backward_close(host(a), b, rtol=1e-4 if dtype == np.float32 else 1e-10)
 
 
+@pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
+@pytest.mark.parametrize("N", [1, 3])
+@pytest.mark.parametrize("family", [pytest.param(1, id="general"), pytest.param(0, id="auto")])
+def test_feature_tiled_channel_widths(oracle, C, N, family):
+    """Every lanes-per-pixel variant of the tiled kernels (C = 4 x a power of two, float32),
+    on an image whose pixel count is no multiple of the tile; the general kernels on the same
+    inputs for comparison.  Forward values are bit-identical in both families."""
+    lib = _lib.load()
+    lib.chop_set_kernel_family(family)
+    try:
+        B, H, W, D = 2, 20, 23, 21
+        t = reference_test_case(3, B, N, H, W, C, D, np.float32, seed=C + N)
+        want, want_mask = oracle.feature_aggregate_fwd(*_args(t, FKEYS))
+        mapped, mask = chop.feature_aggregate_raw(*_inputs(t, FKEYS))
+        assert lib.chop_last_kernel_family() == (2 if family == 0 else 1)
+        assert np.array_equal(host(mask), want_mask)
+        assert np.array_equal(host(mapped), want)
+        g = np.random.default_rng(C).normal(size=want.shape).astype(np.float32)
+        want_g = oracle.feature_aggregate_bwd(*_args(t, FKEYS), g, want_mask)
+        got_g = chop.feature_aggregate_grad(*_inputs(t, FKEYS), dev(g), mask)
+        assert lib.chop_last_kernel_family() == (2 if family == 0 else 1)
+        for a, b in zip(got_g, want_g):
+            assert_backward_close(host(a), b)
+    finally:
+        lib.chop_set_kernel_family(0)
+
+
 def test_feature_autograd_and_errors(oracle):
     t = reference_test_case(3, 1, 2, 8, 10, 4, 5, np.float64, seed=6)
     ins = _inputs(t, FKEYS)
@@ -210,7 +237,24 @@ def test_full_size_benchmark_tensors(oracle):
         assert np.array_equal(host(mask), want_mask)
         assert np.array_equal(host(cost), want_cost)
         del cost, mask
-    mapped, fmask = chop.feature_aggregate_raw(*[ins[k] for k in (1, 2, 3, 4, 5)])
+    fin = [ins[k] for k in (1, 2, 3, 4, 5)]
+    mapped, fmask = chop.feature_aggregate_raw(*fin)
+    assert _lib.load().chop_last_kernel_family() == 2
     want, want_mask = oracle.feature_aggregate_fwd(*_args(t, FKEYS), threads=16)
     assert np.array_equal(host(fmask), want_mask)
     assert np.array_equal(host(mapped), want)
+    del mapped, want
+    # gradient at full size: linearity in the upstream gradient and the known total
+    # (every accepted sample's four weights sum to 1, so sum(src_grad) = sum of the
+    # upstream gradient over accepted samples)
+    g = torch.randn(1, 128, 160, 192, 2, 32, device="cuda")
+    sg, bg = chop.feature_aggregate_grad(*fin, g, fmask)
+    assert _lib.load().chop_last_kernel_family() == 2
+    total = (g.double() * fmask.double()).sum().item()
+    assert abs(sg.double().sum().item() - total) < 1e-6 * g.double().abs().sum().item()
+    sg2, bg2 = chop.feature_aggregate_grad(*fin, 2 * g, fmask)
+    assert_backward_close(host(sg2), 2 * host(sg))
+    assert_backward_close(host(bg2), 2 * host(bg))
+    want_sg, want_bg = oracle.feature_aggregate_bwd(*_args(t, FKEYS), host(g), want_mask)
+    assert_backward_close(host(sg), want_sg)
+    assert_backward_close(host(bg), want_bg)
