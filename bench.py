@@ -5,8 +5,9 @@ synthetic input that is already resident in HBM.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2] [--no-cpu-baseline]
 
-The default run is the headline configuration (workload 2, MEAN).  ``--reduce MIN`` and
-``--aggregate`` (CostAggregate on the same tensors, float32 workloads only) time the other
+The default run is the headline configuration (workload 2, MEAN).  ``--reduce MIN``,
+``--aggregate`` (CostAggregate), ``--v3 GROUPS`` (CostVolumeV3) and ``--feature``
+(FeatureAggregate), all on the same tensors and for float32 workloads only, time the other
 entry points for the tables under profiles/.
 """
 import argparse
@@ -37,6 +38,7 @@ class Runner:
         self.Rs, self.Ts = up("Rs"), up("Ts")
         self.v2 = wl.op == "v2"
         self.agg = wl.op == "agg"
+        self.v3, self.feat = wl.op == "v3", wl.op == "feat"
         self.red = 0 if wl.reduce_method == "MEAN" else 1
         if self.v2:
             self.depth_grid = up("depth_grid")
@@ -44,8 +46,8 @@ class Runner:
             self.base_plane, self.offsets = up("base_plane"), up("offsets")
         B, H, W, D, OC = wl.B, wl.H, wl.W, wl.D, wl.out_channels
         self.cost = torch.empty((B, H, W, D, OC), dtype=td, device=d)
-        self.mask = torch.empty((B, H, W, D, 1 if self.red == 0 else OC), dtype=torch.int32,
-                                device=d)
+        mask_last = wl.N if self.feat else 1 if self.red == 0 else 3 if self.v3 else OC
+        self.mask = torch.empty((B, H, W, D, mask_last), dtype=torch.int32, device=d)
         gen = torch.Generator(device=d)
         gen.manual_seed(wl.seed)
         self.cost_grad = torch.randn((B, H, W, D, OC), dtype=torch.float32, device=d,
@@ -80,6 +82,15 @@ class Runner:
             rc = lib.chop_cost_aggregate_fwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
                                                  p(self.base_plane), p(self.offsets), p(self.Rs),
                                                  p(self.Ts), p(self.cost), p(self.mask))
+        elif self.v3:
+            rc = lib.chop_cost_volume_v3_fwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
+                                                 p(self.ref), p(self.src), p(self.base_plane),
+                                                 p(self.offsets), p(self.Rs), p(self.Ts),
+                                                 p(self.cost), p(self.mask))
+        elif self.feat:
+            rc = lib.chop_feature_aggregate_fwd_f32(s, 1, *self.dims, p(self.src),
+                                                    p(self.base_plane), p(self.offsets), p(self.Rs),
+                                                    p(self.Ts), p(self.cost), p(self.mask))
         elif self.storage_code:
             rc = lib.chop_cost_volume_fwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
@@ -110,6 +121,15 @@ class Runner:
             rc = lib.chop_cost_aggregate_bwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
                                                  p(self.base_plane), p(self.offsets), p(self.Rs),
                                                  p(self.Ts), *tail)
+        elif self.v3:
+            rc = lib.chop_cost_volume_v3_bwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
+                                                 p(self.ref), p(self.src), p(self.base_plane),
+                                                 p(self.offsets), p(self.Rs), p(self.Ts), *tail)
+        elif self.feat:
+            rc = lib.chop_feature_aggregate_bwd_f32(s, 1, *self.dims, p(self.src),
+                                                    p(self.base_plane), p(self.offsets), p(self.Rs),
+                                                    p(self.Ts), p(self.cost_grad), p(self.mask),
+                                                    p(self.src_grad), p(self.depth_grad))
         elif self.storage_code:
             rc = lib.chop_cost_volume_bwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
@@ -155,6 +175,16 @@ def cpu_baseline(wl, budget_s=12.0):
             args = (ref, src, bp, t["offsets"], t["Rs"], t["Ts"])
             _, mask = oracle.cost_aggregate_fwd(*args, wl.reduce_method, threads=threads)
             oracle.cost_aggregate_bwd(*args, cg[..., 0], mask, wl.reduce_method, threads=threads)
+        elif wl.op == "v3":
+            bp = t["base_plane"][:, sl]
+            args = (ref, src, bp, t["offsets"], t["Rs"], t["Ts"])
+            _, mask = oracle.cost_volume_v3_fwd(*args, wl.reduce_method, wl.groups, threads=threads)
+            oracle.cost_volume_v3_bwd(*args, cg, mask, wl.reduce_method, wl.groups)
+        elif wl.op == "feat":
+            bp = t["base_plane"][:, sl]
+            args = (src, bp, t["offsets"], t["Rs"], t["Ts"])
+            _, mask = oracle.feature_aggregate_fwd(*args, threads=threads)
+            oracle.feature_aggregate_bwd(*args, cg.reshape(wl.B, rows, wl.W, wl.D, wl.N, wl.C), mask)
         else:
             dg = t["depth_grid"][:, sl]
             args = (ref, src, dg, t["Rs"], t["Ts"])
@@ -181,6 +211,10 @@ def main():
     ap.add_argument("--reduce", choices=["MEAN", "MIN"], default="MEAN")
     ap.add_argument("--aggregate", action="store_true",
                     help="time CostAggregate on the workload's tensors (float32 CostVolume workloads)")
+    ap.add_argument("--v3", type=int, default=0, metavar="GROUPS",
+                    help="time CostVolumeV3 with this many channel groups on the workload's tensors")
+    ap.add_argument("--feature", action="store_true",
+                    help="time FeatureAggregate on the workload's tensors")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
@@ -198,6 +232,11 @@ def main():
         if wl.op != "v1" or wl.storage != "f32":
             sys.exit("bench.py: --aggregate needs a float32 CostVolume workload (1, 2 or 5)")
         wl.op = "agg"
+    if a.v3 or a.feature:
+        if wl.op != "v1" or wl.storage != "f32":
+            sys.exit("bench.py: --v3 / --feature need a float32 CostVolume workload (1, 2 or 5)")
+        wl.op = "v3" if a.v3 else "feat"
+        wl.groups = a.v3 if a.v3 else 1
     r = Runner(wl, torch, lib)
     ev = lambda: torch.cuda.Event(enable_timing=True)
     for _ in range(a.warmup):
@@ -234,7 +273,7 @@ def main():
     traffic = None
     try:  # measured with rocprofv3 counters in a separate run; the summary is under profiles/
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            t = json.load(f)[wl.name if wl.op != "agg" and a.reduce == "MEAN" else "-"][dominant]
+            t = json.load(f)[wl.name if wl.op in ("v1", "v2") and a.reduce == "MEAN" else "-"][dominant]
         traffic = t["fetch_bytes"] + t["write_bytes"]
     except (OSError, KeyError, ValueError):
         pass
@@ -246,9 +285,10 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": wl.storage, "data": "synthetic",
         "config": {"workload": "%s: %s B%d N%d %dx%d C%d D%d%s %s fwd+bwd" % (
-            wl.name, {"v1": "CostVolume", "v2": "CostVolumeV2", "agg": "CostAggregate"}[wl.op],
+            wl.name, {"v1": "CostVolume", "v2": "CostVolumeV2", "agg": "CostAggregate", "v3": "CostVolumeV3",
+                      "feat": "FeatureAggregate"}[wl.op],
             wl.B, wl.N, wl.H, wl.W,
-            wl.C, wl.D, " G%d" % wl.groups if wl.op == "v2" else "", wl.storage),
+            wl.C, wl.D, " G%d" % wl.groups if wl.op in ("v2", "v3") else "", wl.storage),
             "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,

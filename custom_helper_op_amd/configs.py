@@ -23,6 +23,8 @@ class Workload:
     op: str                # "v1": CostVolume (base_plane + offsets, squared difference)
                            # "v2": CostVolumeV2 (depth_grid, group-wise correlation)
                            # "agg": CostAggregate (v1's inputs, channels summed: one value/voxel)
+                           # "v3": CostVolumeV3 (v1's inputs, best group pair: one value/voxel)
+                           # "feat": FeatureAggregate (v1's inputs without ref: N*C values/voxel)
     storage: str           # element type of ref/src/cost/cost_grad: f32, f64, f16, bf16
     B: int
     N: int
@@ -43,7 +45,9 @@ class Workload:
 
     @property
     def out_channels(self) -> int:
-        return self.groups if self.op == "v2" else 1 if self.op == "agg" else self.C
+        if self.op == "feat":
+            return self.N * self.C
+        return self.groups if self.op == "v2" else 1 if self.op in ("agg", "v3") else self.C
 
     def elem_bytes(self) -> int:
         return {"f32": 4, "f64": 8, "f16": 2, "bf16": 2}[self.storage]
@@ -70,6 +74,11 @@ class Workload:
         mask = self.voxels * 4 * (1 if self.reduce_method == "MEAN" else self.out_channels)
         if self.op == "agg":
             cost = self.voxels * e  # one value per voxel
+        if self.op == "v3":         # mask: view count, or (view, reference group, source group)
+            mask = self.voxels * 4 * (1 if self.reduce_method == "MEAN" else 3)
+        if self.op == "feat":       # no reference image; one mask entry per (voxel, view)
+            ref = 0
+            mask = self.voxels * self.N * 4
         fwd = ref + src + depth_in + cams + cost + mask
         bwd = ref + src + depth_in + cams + cost + mask + ref + src + depth_grad
         return fwd, bwd

@@ -127,7 +127,7 @@ def _golden_cases():
 
 def test_oracle_reproduces_golden_vectors(oracle):
     blob, names = _golden_cases()
-    assert len(names) == 20
+    assert len(names) == 28
     for name in names:
         op, red, groups, half = (int(x) for x in blob[name + "/attrs"])
         t = {k.split("/")[-1]: blob[k] for k in blob.files if k.startswith(name + "/in/")}
@@ -140,13 +140,22 @@ def test_oracle_reproduces_golden_vectors(oracle):
             a = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
             cost, mask = oracle.cost_aggregate_fwd(*a, red_s, bool(half))
             grads = oracle.cost_aggregate_bwd(*a, t["cost_grad"], mask, red_s, bool(half))
+        elif op == 3:
+            a = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+            cost, mask = oracle.cost_volume_v3_fwd(*a, red_s, groups, bool(half))
+            grads = oracle.cost_volume_v3_bwd(*a, t["cost_grad"], mask, red_s, groups, bool(half))
+        elif op == 4:
+            a = (t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+            cost, mask = oracle.feature_aggregate_fwd(*a, bool(half))
+            grads = oracle.feature_aggregate_bwd(*a, t["cost_grad"], mask, bool(half))
         else:
             a = (t["ref"], t["src"], t["depth_grid"], t["Rs"], t["Ts"])
             cost, mask = oracle.cost_volume_v2_fwd(*a, red_s, groups, bool(half))
             grads = oracle.cost_volume_v2_bwd(*a, t["cost_grad"], mask, red_s, groups, bool(half))
         assert np.array_equal(cost, blob[name + "/out/cost"]), name
         assert np.array_equal(mask, blob[name + "/out/mask"]), name
-        for k, g in zip(("ref_grad", "src_grad", "depth_grad"), grads):
+        keys = ("src_grad", "depth_grad") if op == 4 else ("ref_grad", "src_grad", "depth_grad")
+        for k, g in zip(keys, grads):
             assert np.array_equal(g, blob[name + "/out/" + k]), (name, k)
 
 

@@ -350,18 +350,28 @@ def test_golden_vectors(family):
             cost, mask = chop.cost_aggregate_raw(*ins, red_s, bool(half))
             got = chop.cost_aggregate_grad(*ins, dev(t["cost_grad"]), dev(want_mask), red_s,
                                            bool(half))
+        elif op == 3:
+            ins = [dev(t[k]) for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts")]
+            cost, mask = chop.cost_volume_v3_raw(*ins, red_s, groups, bool(half))
+            got = chop.cost_volume_grad_v3(*ins, dev(t["cost_grad"]), dev(want_mask), red_s, groups,
+                                           bool(half))
+        elif op == 4:
+            ins = [dev(t[k]) for k in ("src", "base_plane", "offsets", "Rs", "Ts")]
+            cost, mask = chop.feature_aggregate_raw(*ins, bool(half))
+            got = chop.feature_aggregate_grad(*ins, dev(t["cost_grad"]), dev(want_mask), bool(half))
         else:
             ins = [dev(t[k]) for k in ("ref", "src", "depth_grid", "Rs", "Ts")]
             cost, mask = chop.cost_volume_v2_raw(*ins, red_s, groups, bool(half))
             got = chop.cost_volume_grad_v2(*ins, dev(t["cost_grad"]), dev(want_mask), red_s, groups,
                                            bool(half))
         assert np.array_equal(host(mask), want_mask), name
-        if family == 1:
+        if family == 1 or op >= 3:   # literal operation order: same bits
             assert np.array_equal(host(cost), want_cost), name
         else:
             assert_forward_close(host(cost), want_cost, atol=1e-5 if op == 1 else 1e-6)
         tol = 1e-4 if want_cost.dtype == np.float32 else 1e-10
-        for g, k in zip(got, ("ref_grad", "src_grad", "depth_grad")):
+        keys = ("src_grad", "depth_grad") if op == 4 else ("ref_grad", "src_grad", "depth_grad")
+        for g, k in zip(got, keys):
             assert_backward_close(host(g), blob[name + "/out/" + k], tol)
 
 
