@@ -31,6 +31,9 @@ for _t in ("f32", "f64"):
     SIGNATURES["chop_cost_volume_v3_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 11
     SIGNATURES["chop_feature_aggregate_fwd_" + _t] = [_vp, _int] + _DIMS + [_vp] * 7
     SIGNATURES["chop_feature_aggregate_bwd_" + _t] = [_vp, _int] + _DIMS + [_vp] * 9
+    SIGNATURES["chop_cost_default_fill_" + _t] = [_vp, _int, _i64, _i64] + [_vp] * 4
+    SIGNATURES["chop_cost_default_fill_grad_" + _t] = [_vp, _int, _i64, _i64] + [_vp] * 4
+    SIGNATURES["chop_combine_projection_" + _t] = [_vp, _i64, _i64] + [_vp] * 5
     SIGNATURES["chop_cost_volume_sample_coords_" + _t] = [_vp, _int] + [_i64] * 7 + [_vp] * 10
 SIGNATURES["chop_cost_volume_fwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 9
 SIGNATURES["chop_cost_volume_bwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 13 + [ctypes.c_size_t]

@@ -457,6 +457,61 @@ V3_ENTRY(f32, float)
 V3_ENTRY(f64, double)
 #undef V3_ENTRY
 
+#define EPILOGUE_ENTRY(SFX, T)                                                                  \
+  int chop_cost_default_fill_##SFX(void *stream, int reduce, int64_t mask_count, int64_t inner, \
+                                   const T *cost, const int32_t *mask, const T *default_cost,   \
+                                   T *out) {                                                    \
+    if (reduce != CHOP_REDUCE_MEAN && reduce != CHOP_REDUCE_MIN)                                \
+      return fail(CHOP_ERR_BAD_ENUM, "reduce must be CHOP_REDUCE_MEAN (0) or CHOP_REDUCE_MIN (1)"); \
+    int64_t total;                                                                              \
+    if (mask_count < 0 || inner < 1 || mul_overflows({mask_count, inner}, &total))              \
+      return fail(CHOP_ERR_BAD_DIMS, "mask_count must be >= 0 and inner >= 1");                 \
+    if (total == 0) return CHOP_OK;                                                             \
+    REQUIRE_PTR(cost, total);                                                                   \
+    REQUIRE_PTR(mask, total);                                                                   \
+    REQUIRE_PTR(default_cost, total);                                                           \
+    REQUIRE_PTR(out, total);                                                                    \
+    return launch_status(launch_default_fill<T>(reduce, mask_count, inner, cost, mask,          \
+                                                default_cost, out,                              \
+                                                static_cast<hipStream_t>(stream)),              \
+                         "default fill launch");                                                \
+  }                                                                                             \
+  int chop_cost_default_fill_grad_##SFX(void *stream, int reduce, int64_t mask_count,           \
+                                        int64_t inner, const T *out_grad, const int32_t *mask,  \
+                                        T *cost_grad, T *default_grad) {                        \
+    if (reduce != CHOP_REDUCE_MEAN && reduce != CHOP_REDUCE_MIN)                                \
+      return fail(CHOP_ERR_BAD_ENUM, "reduce must be CHOP_REDUCE_MEAN (0) or CHOP_REDUCE_MIN (1)"); \
+    int64_t total;                                                                              \
+    if (mask_count < 0 || inner < 1 || mul_overflows({mask_count, inner}, &total))              \
+      return fail(CHOP_ERR_BAD_DIMS, "mask_count must be >= 0 and inner >= 1");                 \
+    REQUIRE_PTR(default_grad, 1);                                                               \
+    REQUIRE_PTR(out_grad, total);                                                               \
+    REQUIRE_PTR(mask, total);                                                                   \
+    REQUIRE_PTR(cost_grad, total);                                                              \
+    return launch_status(launch_default_fill_grad<T>(reduce, mask_count, inner, out_grad, mask, \
+                                                     cost_grad, default_grad,                   \
+                                                     static_cast<hipStream_t>(stream)),         \
+                         "default fill gradient launch");                                       \
+  }                                                                                             \
+  int chop_combine_projection_##SFX(void *stream, int64_t B, int64_t N, const T *ref_cam,       \
+                                    const T *src_cam, const T *scale, T *Rs, T *Ts) {           \
+    int64_t total;                                                                              \
+    if (B < 0 || N < 0 || mul_overflows({B, N, 32}, &total))                                    \
+      return fail(CHOP_ERR_BAD_DIMS, "B and N must be >= 0");                                   \
+    if (total == 0) return CHOP_OK;                                                             \
+    REQUIRE_PTR(ref_cam, total);                                                                \
+    REQUIRE_PTR(src_cam, total);                                                                \
+    REQUIRE_PTR(scale, total);                                                                  \
+    REQUIRE_PTR(Rs, total);                                                                     \
+    REQUIRE_PTR(Ts, total);                                                                     \
+    return launch_status(launch_combine_projection<T>(B, N, ref_cam, src_cam, scale, Rs, Ts,    \
+                                                      static_cast<hipStream_t>(stream)),        \
+                         "combine_projection launch");                                          \
+  }
+EPILOGUE_ENTRY(f32, float)
+EPILOGUE_ENTRY(f64, double)
+#undef EPILOGUE_ENTRY
+
 size_t chop_cost_volume_bwd16_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C,
                                               int64_t N, int64_t srcH, int64_t srcW) {
   if (B < 0 || H < 0 || W < 0 || C < 0 || N < 0 || srcH < 0 || srcW < 0) return 0;

@@ -128,6 +128,19 @@ hipError_t launch_sample_coords(R half, int64_t B, int64_t H, int64_t W, int64_t
                                 R *sw, R *sh, int32_t *fh, int32_t *fw, int32_t *state,
                                 hipStream_t stream);
 
+// CostMapLayer's default fill and its gradient; the relative projection of a camera pair.
+template <typename R>
+hipError_t launch_default_fill(int reduce, int64_t mask_count, int64_t inner, const R *cost,
+                               const int32_t *mask, const R *default_cost, R *out,
+                               hipStream_t stream);
+template <typename R>
+hipError_t launch_default_fill_grad(int reduce, int64_t mask_count, int64_t inner,
+                                    const R *out_grad, const int32_t *mask, R *cost_grad,
+                                    R *default_grad, hipStream_t stream);
+template <typename R>
+hipError_t launch_combine_projection(int64_t B, int64_t N, const R *ref_cam, const R *src_cam,
+                                     const R *scale, R *Rs, R *Ts, hipStream_t stream);
+
 int grid_for(int64_t work_items, int block);
 
 }  // namespace chop

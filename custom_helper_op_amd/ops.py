@@ -582,6 +582,87 @@ def feature_aggregate(src_images, base_plane, offsets, Rs, Ts, half_centor=True,
     return _FeatureAggregate.apply(src_images, base_plane, offsets, Rs, Ts, half_centor)
 
 
+class _DefaultFill(torch.autograd.Function):
+    """``tf.where(valid(cost_mask), cost, default_cost)`` with its gradient, as one kernel each
+    way (custom_helper_op/python/layers/custom_layers.py:52-57, :78-83)."""
+
+    @staticmethod
+    def forward(ctx, cost, cost_mask, default_cost, reduce_method):
+        lib = _lib.load()
+        red = _reduce_code(reduce_method)
+        dt, dev = cost.dtype, cost.device
+        _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+        cost = _prep(cost, dt, dev, "cost")
+        cost_mask = _prep(cost_mask, torch.int32, dev, "cost_mask")
+        default_cost = _prep(default_cost, dt, dev, "default_cost")
+        _require(default_cost.numel() == 1, "default_cost must be a scalar")
+        n_mask = cost_mask.numel()
+        _require(n_mask > 0 and cost.numel() % n_mask == 0 or cost.numel() == 0,
+                 "cost_mask must cover cost with a whole number of elements per entry")
+        inner = cost.numel() // n_mask if n_mask else 1
+        out = torch.empty_like(cost)
+        fn = lib.chop_cost_default_fill_f32 if dt == torch.float32 else lib.chop_cost_default_fill_f64
+        _lib.check(fn(_stream(out), red, n_mask, inner, _ptr(cost), _ptr(cost_mask),
+                      _ptr(default_cost), _ptr(out)))
+        ctx.save_for_backward(cost_mask)
+        ctx.attrs = (red, n_mask, inner, default_cost.shape)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        lib = _lib.load()
+        (cost_mask,) = ctx.saved_tensors
+        red, n_mask, inner, dshape = ctx.attrs
+        grad_out = grad_out.contiguous()
+        cost_grad = torch.empty_like(grad_out)
+        default_grad = torch.empty(dshape, dtype=grad_out.dtype, device=grad_out.device)
+        fn = (lib.chop_cost_default_fill_grad_f32 if grad_out.dtype == torch.float32
+              else lib.chop_cost_default_fill_grad_f64)
+        _lib.check(fn(_stream(cost_grad), red, n_mask, inner, _ptr(grad_out), _ptr(cost_mask),
+                      _ptr(cost_grad), _ptr(default_grad)))
+        return cost_grad, None, default_grad, None
+
+
+def cost_default_fill(cost, cost_mask, default_cost, reduce_method="MEAN"):
+    """``where(cost_mask > 0, cost, default_cost)`` for MEAN, ``cost_mask >= 0`` for MIN: what
+    ``CostMapLayer`` / ``CostMapLayerV2`` apply to the op's outputs; differentiable with respect
+    to ``cost`` and the scalar ``default_cost``.  ``cost_mask`` may have one entry per cost
+    element or one per row of the last axis."""
+    return _DefaultFill.apply(cost, cost_mask, default_cost, reduce_method)
+
+
+def combine_projection(ref_cam, src_cam, scale):
+    """The relative projection the ops take, computed on the device
+    (custom_helper_op/python/ops/op_tests/cost_volume_op_test.py:115-134).
+    ``ref_cam [B,2,4,4]`` (or ``[2,4,4]``), ``src_cam [B,N,2,4,4]`` (or ``[2,4,4]``), ``scale [3]``
+    -> ``(Rs [B,N,3,3], Ts [B,N,3])``; the unbatched form returns ``(R [3,3], T [3,1])`` like the
+    reference helper."""
+    lib = _lib.load()
+    single = ref_cam.dim() == 3
+    dt, dev = ref_cam.dtype, ref_cam.device
+    _require(dt in (torch.float32, torch.float64), "dtype must be float32 or float64")
+    if single:
+        _require(tuple(ref_cam.shape) == (2, 4, 4) and tuple(src_cam.shape) == (2, 4, 4),
+                 "cameras must be [2,4,4]")
+        ref_cam, src_cam = ref_cam[None], src_cam[None, None]
+    ref_cam = _prep(ref_cam, dt, dev, "ref_cam")
+    src_cam = _prep(src_cam, dt, dev, "src_cam")
+    scale = _prep(scale, dt, dev, "scale")
+    _require(ref_cam.dim() == 4 and tuple(ref_cam.shape[1:]) == (2, 4, 4), "ref_cam must be [B,2,4,4]")
+    B = ref_cam.shape[0]
+    _require(src_cam.dim() == 5 and src_cam.shape[0] == B and tuple(src_cam.shape[2:]) == (2, 4, 4),
+             "src_cam must be [B,N,2,4,4]")
+    _require(tuple(scale.shape) == (3,), "scale must have 3 entries")
+    N = src_cam.shape[1]
+    Rs = torch.empty((B, N, 3, 3), dtype=dt, device=dev)
+    Ts = torch.empty((B, N, 3), dtype=dt, device=dev)
+    fn = lib.chop_combine_projection_f32 if dt == torch.float32 else lib.chop_combine_projection_f64
+    _lib.check(fn(_stream(Rs), B, N, _ptr(ref_cam), _ptr(src_cam), _ptr(scale), _ptr(Rs), _ptr(Ts)))
+    if single:
+        return Rs[0, 0], Ts[0, 0][:, None]
+    return Rs, Ts
+
+
 def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):
     """Diagnostic: per-(voxel, view) sample coordinates ``[B,H,W,D,N]`` as the kernels
     compute them: ``(sw, sh, fh, fw, state)``."""

@@ -236,6 +236,40 @@ int chop_feature_aggregate_bwd_f64(void *stream, int half_centor, int64_t B, int
                                    const int32_t *mapped_mask, double *src_grad,
                                    double *base_plane_grad);
 
+/* ---- callers on either side of the ops ----------------------------------------------
+ * Default fill: what CostMapLayer / CostMapLayerV2 do with the op's outputs,
+ *   out = where(valid(mask), cost, *default_cost),  valid = mask > 0 (MEAN) or mask >= 0 (MIN)
+ * (custom_helper_op/python/layers/custom_layers.py:52-57 and :78-83; `default_cost` is the
+ * layer's scalar weight and lives in device memory).  cost and out hold mask_count * inner
+ * elements, `inner` consecutive ones per mask entry (CostAggregate: inner 1, mask [B,H,W,D];
+ * CostVolumeV2 MEAN: inner = groups, mask [B,H,W,D,1]; CostVolumeV2 MIN: inner 1, mask
+ * [B,H,W,D,groups]).  out may be the cost buffer itself.
+ * The gradient of that `where`: cost_grad = out_grad where valid and 0 elsewhere,
+ * *default_grad = sum of out_grad where not valid (the entry zeroes it first). */
+int chop_cost_default_fill_f32(void *stream, int reduce, int64_t mask_count, int64_t inner,
+                               const float *cost, const int32_t *mask, const float *default_cost,
+                               float *out);
+int chop_cost_default_fill_f64(void *stream, int reduce, int64_t mask_count, int64_t inner,
+                               const double *cost, const int32_t *mask,
+                               const double *default_cost, double *out);
+int chop_cost_default_fill_grad_f32(void *stream, int reduce, int64_t mask_count, int64_t inner,
+                                    const float *out_grad, const int32_t *mask, float *cost_grad,
+                                    float *default_grad);
+int chop_cost_default_fill_grad_f64(void *stream, int reduce, int64_t mask_count, int64_t inner,
+                                    const double *out_grad, const int32_t *mask,
+                                    double *cost_grad, double *default_grad);
+/* combine_projection (custom_helper_op/python/ops/op_tests/cost_volume_op_test.py:115-134;
+ * the same helper is repeated in the other op tests): the Rs [B,N,3,3] and Ts [B,N,3] the ops
+ * take, from ref_cam [B,2,4,4] and src_cam [B,N,2,4,4] (first 4x4 the extrinsic [R|t], second
+ * the intrinsic K in its upper-left 3x3) and scale [3] (multiplies the rows of both K; then
+ * 0.5 is added to both principal points):
+ *   R = src_K (src_R ref_R^T) ref_K^-1,   T = src_K (src_t - src_R ref_R^T ref_t). */
+int chop_combine_projection_f32(void *stream, int64_t B, int64_t N, const float *ref_cam,
+                                const float *src_cam, const float *scale, float *Rs, float *Ts);
+int chop_combine_projection_f64(void *stream, int64_t B, int64_t N, const double *ref_cam,
+                                const double *src_cam, const double *scale, double *Rs,
+                                double *Ts);
+
 /* ---- 16-bit storage extension --------------------------------------------------------
  * No counterpart in the reference, whose ops register float32 and float64 only
  * (custom_helper_ops.cc:197,234).  ref, src, cost, cost_grad, ref_grad and src_grad

@@ -260,6 +260,43 @@ def feature_aggregate_bwd(src, base_plane, offsets, Rs, Ts, mapped_grad, mapped_
     return src_grad, bp_grad
 
 
+def cost_default_fill(cost, cost_mask, default_cost, reduce="MEAN"):
+    """``tf.where(cost_mask > 0, cost, default)`` (MEAN) / ``cost_mask >= 0`` (MIN), as the
+    reference's layers apply it (custom_helper_op/python/layers/custom_layers.py:52-57, :78-83);
+    the mask broadcasts over a trailing axis of the cost."""
+    valid = (cost_mask > 0) if _REDUCE[reduce] == 0 else (cost_mask >= 0)
+    while valid.ndim < cost.ndim:
+        valid = valid[..., None]
+    return np.where(valid, cost, np.asarray(default_cost, cost.dtype))
+
+
+def cost_default_fill_grad(out_grad, cost_mask, reduce="MEAN"):
+    """Gradient of that ``where``: ``(cost_grad, default_grad)``."""
+    valid = (cost_mask > 0) if _REDUCE[reduce] == 0 else (cost_mask >= 0)
+    while valid.ndim < out_grad.ndim:
+        valid = valid[..., None]
+    valid = np.broadcast_to(valid, out_grad.shape)
+    return np.where(valid, out_grad, 0), np.where(valid, 0, out_grad).sum(dtype=np.float64)
+
+
+def combine_projection(ref_cam, src_cam, scale):
+    """Line-by-line numpy restatement of the reference helper
+    (custom_helper_op/python/ops/op_tests/cost_volume_op_test.py:115-134) for one camera pair:
+    ``ref_cam, src_cam [2,4,4]``, ``scale [3]`` -> ``(R [3,3], T [3,1])``."""
+    ref_R, ref_T = ref_cam[0, :3, :3], ref_cam[0, :3, 3:]
+    ref_K = ref_cam[1, :3, :3] * scale[:, None]
+    src_R, src_T = src_cam[0, :3, :3], src_cam[0, :3, 3:]
+    src_K = src_cam[1, :3, :3] * scale[:, None]
+    ref_K[0, 2] = ref_K[0, 2] + 0.5
+    ref_K[1, 2] = ref_K[1, 2] + 0.5
+    src_K[0, 2] = src_K[0, 2] + 0.5
+    src_K[1, 2] = src_K[1, 2] + 0.5
+    ref_K_inv = np.linalg.inv(ref_K)
+    delta_R = src_R @ ref_R.T
+    delta_T = src_T - delta_R @ ref_T
+    return src_K @ (delta_R @ ref_K_inv), src_K @ delta_T
+
+
 def sample_coords(base_plane, offsets, Rs, Ts, src_hw, half_centor=True, depth_grid=None):
     """Per-(voxel, view) source coordinates ``[B,H,W,D,N]``: (sw, sh, fh, fw, state)."""
     if depth_grid is not None:
