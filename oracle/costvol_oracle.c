@@ -25,6 +25,15 @@
  *       :338-452 CostMeanAggregateGradKernel -> chop_oracle_cost_aggregate_bwd_* (reduce 0)
  *       :454-563 CostMinAggregateGradKernel  -> chop_oracle_cost_aggregate_bwd_* (reduce 1)
  *
+ *   custom_helper_op/cc/kernels/cost_volume_kernels_gpu_v3.cu.cc
+ *       :33-143  CostMeanVolumeV3Kernel      -> chop_oracle_cost_volume_v3_fwd_* (reduce 0)
+ *       :145-261 CostMinVolumeV3Kernel       -> chop_oracle_cost_volume_v3_fwd_* (reduce 1)
+ *       :376-517 CostMeanVolumeGradV3Kernel  -> chop_oracle_cost_volume_v3_bwd_* (reduce 0)
+ *       :519-639 CostMinVolumeGradV3Kernel   -> chop_oracle_cost_volume_v3_bwd_* (reduce 1)
+ *   custom_helper_op/cc/kernels/feature_aggregate_kernels_gpu.cu.cc
+ *       :33-121  FeatureAggregateKernel      -> chop_oracle_feature_aggregate_fwd_*
+ *       :219-326 FeatureAggregateGradKernel  -> chop_oracle_feature_aggregate_bwd_*
+ *
  * Parity status of each function (what pins it is in tests/test_oracle_*.py):
  *   forward MEAN/MIN (V1), MEAN/MAX (V2): pinned by an independent float64 composite that
  *     restates the reference tests' own oracle, by closed-form camera cases, by a
@@ -36,6 +45,16 @@
  *   aggregate backward: MEAN pinned against the pinned cost-volume backward fed the
  *     upstream gradient broadcast over channels and divided by C; both reduces by finite
  *     differences in float64.
+ *   CostVolumeV3 forward: pinned by the composite (all group pairs by einsum, maximum and
+ *     arg-maximum), by brute force including all-negative correlations (the seed survives)
+ *     and exact ties (first pair wins), and by the pinned V2 oracle for one group.
+ *     Backward: by the V2 gradient for one group and by finite differences in float64.
+ *     Where the reference reads out of bounds (no pair above the seed, :495-496) the view
+ *     contributes nothing here; that choice is not a parity claim.
+ *   FeatureAggregate forward: pinned by the composite (also with a source size different
+ *     from the output grid) and, bit for bit, by the pinned V2 oracle against a reference
+ *     image of ones with one channel per group.  Backward: by that V2 gradient and by
+ *     finite differences.
  *   sample_coords: pinned by the float64 composite's coordinates.
  *   NOT pinned: the rounding of a CUDA build of the reference (nvcc contracts a*b+c into
  *     fused multiply-adds and the reference is built with ftz=true).  No such build or
