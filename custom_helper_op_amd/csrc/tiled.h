@@ -369,6 +369,10 @@ template <int NV>
 constexpr int forward_lds_words(int lpp) {
   return lpp > 1 ? NV * 64 * 5 : 0;
 }
+// The minimum of the summed squared difference also stages one chunk of squares per view:
+// a row of C (+4 padding, so that the eight readers of a pixel hit different banks) floats
+// per (pixel, depth).
+constexpr int forward_squares_words(int lpp) { return lpp > 1 ? 64 * (4 * lpp + 4) : 0; }
 
 // REDUCE: 0 mean over the accepted views (mask = their number), 1 per-channel minimum of
 // the squared difference / per-group maximum of the correlation with the winning view as
@@ -425,6 +429,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
     // ---- phase 1: reprojection by lane (p, j = cl) --------------------------------------
     int r_off[NV];
     float4 r_wts[NV];
+    unsigned vmask = 0u;  // views accepted for lane (p, j)'s own voxel
     {
       const int d = d0 + t.cl;
       const bool d_ok = d < d_hi;
@@ -437,6 +442,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         hit.k00 = hit.k01 = hit.k11 = hit.k10 = 0.f;
         if (n < N && d_ok) reproject<NV>(cam, n, depth, half, g.src_h_max, g.src_w_max, srcW, C, hit);
         cnt += hit.off >= 0;
+        if constexpr (CORR == 2 && REDUCE == 1) vmask |= (hit.off >= 0 ? 1u : 0u) << n;
         if constexpr (CORR == 4) {
           if (n < N && d_ok && t.pix_ok)
             __builtin_nontemporal_store(hit.off >= 0 ? 1 : 0, a.mask + (t.pix * D + d) * N + n);
@@ -454,6 +460,90 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
     }
     if constexpr (LPP > 1) wave_sync();
+    if constexpr (CORR == 2 && REDUCE == 1) {
+      // Minimum over the views of the squared difference summed over ALL channels
+      // (cost_aggregate_kernels_gpu.cu.cc:128-229).  The mask names the winning view, so the
+      // sum has to be the reference's: channel 0 first, every product and sum rounded
+      // separately.  View by view, the channel lanes leave the chunk's squares in LDS and the
+      // lane that owns voxel (p, d0 + cl) adds its row up in channel order.
+      constexpr int kSq = NV * 64 * 20;             // behind the records
+      constexpr int ROWB = (VEC * LPP + 4) * 4;     // bytes per (pixel, depth) row
+      float best = 3.402823466e+38f;                // numeric_limits<T>::max(), :170
+      int win = -1;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        float own = 0.f;  // LPP == 1: this lane holds the whole pixel
+#pragma unroll
+        for (int jj = 0; jj < LPP; ++jj) {
+          if (d0 + jj >= d_hi) {
+            if constexpr (LPP >= 16) continue; else break;
+          }
+          int off;
+          float4 wt;
+          if constexpr (LPP > 1) {
+            off = lds_at<int>(smem, p4, kOff + ((n * LPP + jj) * PPW) * 4);
+            wt = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj) * PPW) * 16);
+          } else {
+            off = r_off[n];
+            wt = r_wts[n];
+          }
+          float sq[VEC];
+#pragma unroll
+          for (int c = 0; c < VEC; ++c) sq[c] = 0.f;
+          if (off >= 0) {
+            if (off != cur[n]) {
+              cur[n] = off;
+              const S *q = view[n] + off;
+              load_vec<S, VEC, false>(q, tap[n][0]);
+              load_vec<S, VEC, false>(q + C, tap[n][1]);
+              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
+              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
+            }
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+              const float smp = wt.x * tap[n][0][c] + wt.y * tap[n][1][c] + wt.z * tap[n][2][c] +
+                                wt.w * tap[n][3][c];
+              const float diff = smp - ref[c];
+              sq[c] = diff * diff;
+            }
+          }
+          if constexpr (LPP > 1) {
+            lds_at<float4>(smem, (unsigned)(t.p * LPP * ROWB + t.cl * VEC * 4), kSq + jj * ROWB) =
+                make_float4(sq[0], sq[1], sq[2], sq[3]);
+          } else {
+            own = 0.f;
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) own += sq[c];
+          }
+        }
+        if constexpr (LPP > 1) {
+          wave_sync();
+          if ((vmask >> n) & 1u) {
+            float tot = 0.f;
+#pragma unroll
+            for (int k = 0; k < LPP; ++k) {
+              const float4 v = lds_at<float4>(
+                  smem, (unsigned)((t.p * LPP + t.cl) * ROWB), kSq + k * VEC * 4);
+              tot += v.x;
+              tot += v.y;
+              tot += v.z;
+              tot += v.w;
+            }
+            if (best > tot) best = tot, win = n;  // strict: the earliest view keeps a tie (:217)
+          }
+          wave_sync();
+        } else {
+          if (((vmask >> n) & 1u) && best > own) best = own, win = n;
+        }
+      }
+      const int d = d0 + t.cl;
+      if (d < d_hi && t.pix_ok) {
+        const float out = win >= 0 ? best / static_cast<float>(C) : 0.f;  // :222-227
+        __builtin_nontemporal_store(out, reinterpret_cast<float *>(a.cost) + t.pix * D + d);
+        __builtin_nontemporal_store(win, a.mask + t.pix * D + d);
+      }
+      continue;
+    }
     float agg_out = 0.f;
     // ---- phase 2: channel arithmetic by lane (p, channel slice) ---------------------------
 #pragma unroll

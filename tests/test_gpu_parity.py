@@ -500,11 +500,11 @@ def test_tiled_channel_widths(oracle, C, N):
         _assert_family(0)
         for g, w in zip(got, want):
             assert_backward_close(host(g), w)
-        # minimum of the summed squared difference: forward on the general kernel (the sum
-        # must follow the reference's channel order to name the same winner), backward tiled
+        # minimum of the summed squared difference: the tiled forward adds the channels in
+        # the reference's order (staged through LDS), so winner and cost are bit-exact
         want_cost, want_mask = oracle.cost_aggregate_fwd(*args, "MIN")
         cost, mask = chop.cost_aggregate_raw(*_v1_inputs(t), "MIN")
-        _assert_family(1)
+        _assert_family(0)
         assert np.array_equal(host(mask), want_mask) and np.array_equal(host(cost), want_cost)
         cg = rng.standard_normal(want_cost.shape).astype(np.float32)
         want = oracle.cost_aggregate_bwd(*args, cg, want_mask, "MIN")
