@@ -767,7 +767,8 @@ constexpr int backward_record_words() {
 template <int VEC, int LPP, int NV>
 constexpr int backward_lds_words() {
   using WN = Window<VEC, LPP>;
-  return backward_record_words<VEC, LPP, NV>() + NV * WN::SLOTS * WN::STRIDE;
+  // records (or list), windows, and one cell (4 texels x C) staged on its way to memory
+  return backward_record_words<VEC, LPP, NV>() + NV * WN::SLOTS * WN::STRIDE + 4 * WN::C;
 }
 
 // Minimum over the 64 lanes, in registers: four DPP steps reduce each row of 16 lanes,
@@ -883,21 +884,62 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
           __hip_atomic_fetch_add(d + i, v[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
       }
     }
-  } else {
-    // the cell sticks out of the window (samples jumping far apart): add to memory
-    const int fh = key >> 16, fw = key & 0xffff;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int y = fh + (k >> 1), x = fw + ((k == 1 || k == 2) ? 1 : 0);
-      float *gp = gview + (int64_t)(y * srcW + x) * WN::C + cl * VEC;
-#pragma unroll
-      for (int i = 0; i < VEC; ++i) atomic_add(gp + i, v[k][i]);
-    }
   }
+  // (a cell that sticks out of the window never gets here: flush_cells_to_memory took it)
 #pragma unroll
   for (int k = 0; k < 4; ++k)
 #pragma unroll
     for (int i = 0; i < VEC; ++i) v[k][i] = 0.f;
+}
+
+// Cells that stick out of the window (samples of consecutive depths jumping far apart, as
+// they do close to the cameras) go to memory directly.  Uniform control flow: `m` has the
+// lane bits of every pixel with such a cell (`mine` for the caller's own lanes).  One pixel
+// at a time, its lanes lay the four tap images out in LDS as two rows of two adjacent texels
+// and the whole wave adds each row as a dense run of 2*C consecutive floats.  Added lane by
+// lane from the registers, each 16-byte chunk of a texel would carry one float per
+// instruction, and the atomics cost per chunk, not per float.
+template <int VEC, int LPP>
+__device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool mine, int key,
+                                                      float (&v)[4][VEC], float *stage,
+                                                      float *gview, int srcW, int lane, int cl) {
+  constexpr int C = VEC * LPP;
+  typedef float vecf __attribute__((ext_vector_type(VEC)));
+  while (m) {
+    const int lead = __ffsll((long long)m) - 1;
+    m &= ~(((1ull << LPP) - 1ull) << lead);
+    const int k2 = __builtin_amdgcn_readlane(key, lead);  // the same in all lanes of the pixel
+    if (lane - cl == lead) {
+      // taps 00, 01 (row fh), then 10, 11 (row fh + 1); v is ordered 00, 01, 11, 10
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        vecf w;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) w[i] = v[k][i];
+        *reinterpret_cast<vecf *>(stage + (k == 2 ? 3 : k == 3 ? 2 : k) * C + cl * VEC) = w;
+      }
+    }
+    wave_sync();
+    const int fh = k2 >> 16, fw = k2 & 0xffff;
+    float *row0 = gview + (int64_t)(fh * srcW + fw) * C;
+    float *row1 = row0 + (int64_t)srcW * C;
+#pragma unroll
+    for (int f0 = 0; f0 < 2 * C; f0 += 64) {
+      const int f = f0 + lane;
+      if (f < 2 * C) {
+        const float a0 = stage[f], a1 = stage[2 * C + f];
+        if (a0 != 0.f) atomic_add(row0 + f, a0);
+        if (a1 != 0.f) atomic_add(row1 + f, a1);
+      }
+    }
+    wave_sync();
+  }
+  if (mine) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[k][i] = 0.f;
+  }
 }
 
 // Waves per SIMD the register budget is held to.  The kernel is latency-bound (its time
@@ -930,6 +972,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   int *s_list = NV == 1 ? reinterpret_cast<int *>(smem)
                         : reinterpret_cast<int *>(smem) + (LPP > 1 ? NV * 64 * 11 + 128 : 0);
   float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV>();
+  float *s_stage = s_data + NV * WN::SLOTS * WN::STRIDE;
   for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
 
   Cameras<NV> cam;
@@ -1014,6 +1057,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     int2 r_cell[NV];
     float r_scl = 0.f;
     float4 r_wts[NV], r_dwt[NV];
+    bool chunk_out[NV];  // some cell of this chunk (or the open one) sticks out of the window
     // Issue the loads of this chunk's cost_grad rows now, unconditionally, so that the
     // reprojection below overlaps their latency.  Streaming loads: cached ones let the
     // next view's workgroup hit L2 more often (690 -> 660 MB fetched) and save 10 us here,
@@ -1094,6 +1138,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         // their bounding box, and whatever still sticks out is marked for the memory path.
         const bool valid = hit.off >= 0;
         bool in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
+        chunk_out[n] = false;
         if (__ballot(!(in_new && (cur[n] < 0 || cell[n].y < 0))) != 0ull) {
           int my = WN::kNone, mx = WN::kNone, My = -WN::kNone, Mx = -WN::kNone;
           if (valid) my = My = hit.key >> 16, mx = Mx = hit.key & 0xffff;
@@ -1110,6 +1155,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
           const int ck = cell[n].y & 0x7fffffff;
           cell[n].y = WN::inside(ck, oy[n], ox[n]) ? (ck | WN::kInside) : ck;
+          chunk_out[n] = __ballot((valid && !in_new) || (cur[n] >= 0 && cell[n].y >= 0)) != 0ull;
         }
         const int2 rec = make_int2(WN::kPacked ? (int)WN::pack_slots(hit.key) : 0,
                                    (valid && in_new) ? (hit.key | WN::kInside) : hit.key);
@@ -1180,6 +1226,20 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       const float4 *rec_wt = rb_wt[cb], *rec_dwt = rb_dwt[cb];
       const float scl = rb_scl[cb];
       float dvox = 0.f;  // this lane's share of d(loss)/d(depth of this voxel)
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        if (chunk_out[n]) {  // uniform, and false for the whole chunk in the usual case
+          // runs that end at this depth on a cell outside the window: to memory, now
+          const bool fire_out = scl != 0.f && rec_off[n] >= 0 && rec_off[n] != cur[n] &&
+                                cur[n] >= 0 && cell[n].y >= 0;
+          const unsigned long long m = __ballot(fire_out);
+          if (m != 0ull) {
+            flush_cells_to_memory<VEC, LPP>(m, fire_out, cell[n].y, sg[n], s_stage, gview[n], srcW,
+                                            t.lane, t.cl);
+            if (fire_out) cur[n] = -1;
+          }
+        }
+      }
       if (scl != 0.f) {
         float cg[VEC];
         {
@@ -1220,6 +1280,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           const float4 wt = rec_wt[n], dwt = rec_dwt[n];
           if (off >= 0) {
             if (off != cur[n]) {
+              // (a run whose cell sticks out of the window was closed by the uniform block
+              // above, which left cur[n] = -1)
               // the run on the previous cell ends.  Start fetching the new cell's taps
               // first, then hand the old cell's image to the window while they arrive.
               // byte offsets in 32 bits: the loads take the view's base from scalar registers
@@ -1307,7 +1369,12 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   // the runs still open, then everything the windows hold
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
-    if (cur[n] >= 0)
+    const bool out = cur[n] >= 0 && cell[n].y >= 0;
+    const unsigned long long m = __ballot(out);
+    if (m != 0ull)
+      flush_cells_to_memory<VEC, LPP>(m, out, cell[n].y, sg[n], s_stage, gview[n], srcW, t.lane,
+                                      t.cl);
+    if (cur[n] >= 0 && !out)
       window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
                            s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW, t.lane, t.cl);
   }
