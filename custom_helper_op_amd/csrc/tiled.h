@@ -544,6 +544,141 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       }
       continue;
     }
+    if constexpr ((CORR == 0 || CORR == 1) && (NV >= 5 || (NV >= 3 && LPP == 4))) {
+      // ---- phase 2, one view at a time (many views) ---------------------------------------
+      // With every view's four taps live at once the kernel needs ~25 registers per view
+      // (171 for six views: two waves per SIMD).  Here a block of up to eight depths keeps
+      // its accumulators and the views take turns with one set of taps, so the register count
+      // hardly depends on the number of views.  Every accumulator still receives the views in
+      // order 0..N-1 with the same operations, so the results are those of the
+      // depth-by-depth loop.  (Measurements decide where this form is used: for three or four
+      // views the depth-by-depth loop needs fewer registers at 32+ channels, and with one or
+      // two lanes per pixel its taps, which survive from chunk to chunk, matter more.)
+      constexpr int DB = LPP < 8 ? LPP : 8;
+#pragma unroll
+      for (int j0 = 0; j0 < LPP; j0 += DB) {
+      float acc[DB][VEC];
+      int arg[REDUCE == 1 ? DB : 1][VEC];
+      int kcnt[DB];
+#pragma unroll
+      for (int jj = 0; jj < DB; ++jj) {
+        kcnt[jj] = 0;
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+          acc[jj][c] = REDUCE == 0 ? 0.f : CORR == 0 ? 3.402823466e+38f : 1.175494351e-38f;
+          if constexpr (REDUCE == 1) arg[jj][c] = -1;
+        }
+      }
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        int cur1 = -1;
+        float tp[4][VEC];
+#pragma unroll
+        for (int jj = 0; jj < DB; ++jj) {
+          if (d0 + j0 + jj >= d_hi) continue;
+          int off;  // -1 also for a view beyond N (phase 1 leaves those records empty)
+          if constexpr (LPP > 1)
+            off = lds_at<int>(smem, p4, kOff + ((n * LPP + j0 + jj) * PPW) * 4);
+          else
+            off = r_off[n];
+          if (off < 0) continue;
+          float4 wt;
+          if constexpr (LPP > 1)
+            wt = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + j0 + jj) * PPW) * 16);
+          else
+            wt = r_wts[n];
+          if (off != cur1) {
+            cur1 = off;
+            const S *q = view[n] + off;
+            load_vec<S, VEC, false>(q, tp[0]);
+            load_vec<S, VEC, false>(q + C, tp[1]);
+            load_vec<S, VEC, false>(q + row_step + C, tp[2]);
+            load_vec<S, VEC, false>(q + row_step, tp[3]);
+          }
+          ++kcnt[jj];
+          if constexpr (REDUCE == 1) {
+            float val[VEC];
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+              const float smp = wt.x * tp[0][c] + wt.y * tp[1][c] + wt.z * tp[2][c] + wt.w * tp[3][c];
+              if (CORR == 0) {
+                const float diff = smp - ref[c];
+                val[c] = diff * diff;
+              } else {
+                val[c] = smp * ref[c];
+              }
+            }
+            if (CORR == 0) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c)
+                if (acc[jj][c] > val[c]) acc[jj][c] = val[c], arg[jj][c] = n;
+            } else {
+#pragma unroll
+              for (int gi = 0; gi < VEC; ++gi) {
+                if (gi * g.sub < VEC) {
+                  float corr = 0.f;
+#pragma unroll
+                  for (int c = 0; c < VEC; ++c)
+                    if (c >= gi * g.sub && c < (gi + 1) * g.sub) corr += val[c];
+                  if (acc[jj][gi] < corr) acc[jj][gi] = corr, arg[jj][gi] = n;
+                }
+              }
+            }
+          } else {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+              if (CORR != 1) {
+                float diff = __builtin_fmaf(wt.x, tp[0][c], -ref[c]);
+                diff = __builtin_fmaf(wt.y, tp[1][c], diff);
+                diff = __builtin_fmaf(wt.z, tp[2][c], diff);
+                diff = __builtin_fmaf(wt.w, tp[3][c], diff);
+                acc[jj][c] = __builtin_fmaf(diff, diff, acc[jj][c]);
+              } else {
+                float smp = wt.x * tp[0][c];
+                smp = __builtin_fmaf(wt.y, tp[1][c], smp);
+                smp = __builtin_fmaf(wt.z, tp[2][c], smp);
+                smp = __builtin_fmaf(wt.w, tp[3][c], smp);
+                acc[jj][c] = __builtin_fmaf(smp, ref[c], acc[jj][c]);
+              }
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < DB; ++jj) {
+        const int d = d0 + j0 + jj;
+        if (d >= d_hi || !t.pix_ok) continue;
+        S *out = a.cost + (t.pix * D + d) * OC;
+        if constexpr (REDUCE == 1) {
+          int32_t *mout = a.mask + (t.pix * D + d) * OC;
+          if (CORR == 0) {
+            store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
+            store_ints<VEC>(mout + t.cl * VEC, arg[jj]);
+          } else {
+            store_groups<S, VEC, true>(out + t.cl * gv, acc[jj], g.sub);
+            if (g.sub == 1) store_ints<VEC>(mout + t.cl * gv, arg[jj]);
+            else if (g.sub == 2) store_ints<VEC / 2>(mout + t.cl * gv, arg[jj]);
+            else store_ints<VEC / 4>(mout + t.cl * gv, arg[jj]);
+          }
+        } else {
+          if (kcnt[jj] > 1) {
+            const float inv = __builtin_amdgcn_rcpf(static_cast<float>(kcnt[jj]));
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) acc[jj][c] *= inv;
+          }
+          if (CORR == 0) {
+            store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
+          } else {
+            float grp[VEC];
+            fold_groups<VEC>(acc[jj], g.sub, grp);
+            store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
+          }
+        }
+      }
+      }  // block of depths
+      if constexpr (LPP > 1) wave_sync();
+      continue;
+    }
     float agg_out = 0.f;
     // ---- phase 2: channel arithmetic by lane (p, channel slice) ---------------------------
 #pragma unroll
