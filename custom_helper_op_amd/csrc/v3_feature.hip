@@ -36,134 +36,7 @@ __device__ __forceinline__ Taps<R> taps_of(const R *src, const Sample<R> &s, int
   return t;
 }
 
-// Best (source group, reference group) pair of one accepted sample: source group outermost,
-// strict "<", seeded with `seed` (cost_volume_kernels_gpu_v3.cu.cc:113-130, 231-250).
-// gi, gs are left untouched when no pair exceeds the seed.
-template <typename R>
-__device__ __forceinline__ R best_pair(const Sample<R> &s, const Taps<R> &t, const R *ref_px,
-                                       int groups, int sub, R seed, int &gi_out, int &gs_out) {
-  R buf[kMaxSubChannels];
-  R best = seed;
-  for (int gs = 0; gs < groups; ++gs) {
-#pragma unroll
-    for (int k = 0; k < kMaxSubChannels; ++k) {
-      if (k < sub) {
-        const int sc = gs * sub + k;
-        buf[k] = s.k00 * t.t00[sc] + s.k01 * t.t01[sc] + s.k11 * t.t11[sc] + s.k10 * t.t10[sc];
-      }
-    }
-    for (int gi = 0; gi < groups; ++gi) {
-      R tmp = R(0);
-#pragma unroll
-      for (int k = 0; k < kMaxSubChannels; ++k)
-        if (k < sub) tmp += buf[k] * ref_px[gi * sub + k];
-      if (best < tmp) {
-        best = tmp;
-        gi_out = gi;
-        gs_out = gs;
-      }
-    }
-  }
-  return best;
-}
-
-template <typename R, int REDUCE>
-__global__ __launch_bounds__(kBlock) void v3_forward_kernel(const Args<R> a) {
-  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  const int groups = a.groups, sub = C / groups;
-  const int64_t total = a.voxels();
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * kBlock) {
-    const Voxel<R> v = locate(a, i);
-    const R *ref_px = a.ref + v.pix * C;
-    R acc = REDUCE == 0 ? R(0) : Limits<R>::min_positive();
-    int used = 0, wn = -1, wgi = -1, wgs = -1;
-    for (int n = 0; n < N; ++n) {
-      Sample<R> s;
-      const int64_t cam = (int64_t)v.b * N + n;
-      project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
-      if (s.state != 2) continue;
-      const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
-      int gi = -1, gs = -1;
-      if (REDUCE == 0) {
-        acc += best_pair(s, t, ref_px, groups, sub, Limits<R>::min_positive(), gi, gs);
-        ++used;
-      } else {
-        const R best = best_pair(s, t, ref_px, groups, sub, acc, gi, gs);
-        if (gi >= 0) {
-          acc = best;
-          wn = n, wgi = gi, wgs = gs;
-        }
-      }
-    }
-    if (REDUCE == 0) {
-      a.mask[i] = used;
-      a.cost[i] = used > 0 ? acc / static_cast<R>(used) : R(0);
-    } else {
-      a.mask[i * 3] = wn, a.mask[i * 3 + 1] = wgi, a.mask[i * 3 + 2] = wgs;
-      a.cost[i] = wn >= 0 ? acc : R(0);
-    }
-  }
-}
-
-template <typename R, int REDUCE>
-__global__ __launch_bounds__(kBlock) void v3_backward_kernel(const Args<R> a) {
-  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  const int groups = a.groups, sub = C / groups;
-  const int64_t total = a.voxels();
-  const int64_t row_step = (int64_t)srcW * C;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * kBlock) {
-    const int32_t *m = a.mask_in + (REDUCE == 0 ? i : i * 3);
-    const int32_t m0 = m[0];
-    if (REDUCE == 0 ? (m0 <= 0) : (m0 < 0)) continue;
-    const Voxel<R> v = locate(a, i);
-    const R *ref_px = a.ref + v.pix * C;
-    R *ref_out = a.ref_grad + v.pix * C;
-    // :426 cost_grad / (T)mask for the mean; the MIN gradient takes cost_grad as is (:621)
-    const R cg = REDUCE == 0 ? a.cost_grad[i] / static_cast<R>(m0) : a.cost_grad[i];
-    R depth_grad = R(0);
-    const int n_lo = REDUCE == 0 ? 0 : m0, n_hi = REDUCE == 0 ? N : m0 + 1;
-    for (int n = n_lo; n < n_hi && n < N; ++n) {
-      Sample<R> s;
-      const int64_t cam = (int64_t)v.b * N + n;
-      project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
-      // A winner that is not accepted any more (inputs changed since the forward pass) is
-      // skipped; the reference would read and write out of bounds (:593-595).
-      if (s.state != 2) continue;
-      const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
-      int gi = -1, gs = -1;
-      if (REDUCE == 0) {
-        best_pair(s, t, ref_px, groups, sub, Limits<R>::min_positive(), gi, gs);
-        // no pair above the seed: the reference indexes group -1 here (:495-496)
-        if (gi < 0) continue;
-      } else {
-        gi = m[1], gs = m[2];
-        if (gi < 0 || gi >= groups || gs < 0 || gs >= groups) continue;
-      }
-      R *g00 = a.src_grad + (t.t00 - a.src);
-      R h_grad = R(0), w_grad = R(0);
-      for (int k = 0; k < sub; ++k) {
-        const int rc = gi * sub + k, cc = gs * sub + k;
-        const R v00 = t.t00[cc], v01 = t.t01[cc], v11 = t.t11[cc], v10 = t.t10[cc];
-        const R smp = s.k00 * v00 + s.k01 * v01 + s.k11 * v11 + s.k10 * v10;
-        atomic_add(ref_out + rc, cg * smp);
-        const R bg = cg * ref_px[rc];
-        atomic_add(g00 + cc, bg * s.k00);
-        atomic_add(g00 + C + cc, bg * s.k01);
-        atomic_add(g00 + C + row_step + cc, bg * s.k11);
-        atomic_add(g00 + row_step + cc, bg * s.k10);
-        const R t1 = v11 - v10 - v01 + v00;
-        h_grad += bg * (t1 * s.dw + v10 - v00);
-        w_grad += bg * (t1 * s.dh + v01 - v00);
-      }
-      depth_grad += depth_chain(s, h_grad, w_grad);
-    }
-    atomic_add(a.depth_grad + v.pix, depth_grad);
-  }
-}
-
-// ---- FeatureAggregate --------------------------------------------------------------------
+// ---- 16-byte slices of a channel row ------------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename R, int VEC>
@@ -196,6 +69,197 @@ __device__ __forceinline__ void store_slice(R *p, const Slice<R, VEC> &in) {
   }
 }
 
+// Best (source group, reference group) pair of one accepted sample: source group outermost,
+// strict "<", seeded with `seed` (cost_volume_kernels_gpu_v3.cu.cc:113-130, 231-250).
+// gi, gs are left untouched when no pair exceeds the seed.
+// SUB: channels per group when that is 4 or 8 floats and every row is 16-byte aligned (the
+// taps and the reference groups are then fetched with 16-byte loads), 0 for any other case.
+// The arithmetic is the same expression per element either way.
+template <typename R, int SUB>
+__device__ __forceinline__ R best_pair(const Sample<R> &s, const Taps<R> &t, const R *ref_px,
+                                       int groups, int sub, R seed, int &gi_out, int &gs_out) {
+  R buf[kMaxSubChannels];
+  R best = seed;
+  for (int gs = 0; gs < groups; ++gs) {
+    if constexpr (SUB > 0) {
+#pragma unroll
+      for (int k0 = 0; k0 < SUB; k0 += 4) {
+        const int sc = gs * SUB + k0;
+        const Slice<R, 4> v00 = load_slice<R, 4>(t.t00 + sc), v01 = load_slice<R, 4>(t.t01 + sc),
+                          v11 = load_slice<R, 4>(t.t11 + sc), v10 = load_slice<R, 4>(t.t10 + sc);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          buf[k0 + k] = s.k00 * v00.v[k] + s.k01 * v01.v[k] + s.k11 * v11.v[k] + s.k10 * v10.v[k];
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kMaxSubChannels; ++k) {
+        if (k < sub) {
+          const int sc = gs * sub + k;
+          buf[k] = s.k00 * t.t00[sc] + s.k01 * t.t01[sc] + s.k11 * t.t11[sc] + s.k10 * t.t10[sc];
+        }
+      }
+    }
+    for (int gi = 0; gi < groups; ++gi) {
+      R tmp = R(0);
+      if constexpr (SUB > 0) {
+#pragma unroll
+        for (int k0 = 0; k0 < SUB; k0 += 4) {
+          const Slice<R, 4> r = load_slice<R, 4>(ref_px + gi * SUB + k0);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) tmp += buf[k0 + k] * r.v[k];
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kMaxSubChannels; ++k)
+          if (k < sub) tmp += buf[k] * ref_px[gi * sub + k];
+      }
+      if (best < tmp) {
+        best = tmp;
+        gi_out = gi;
+        gs_out = gs;
+      }
+    }
+  }
+  return best;
+}
+
+template <typename R, int REDUCE, int SUB>
+__global__ __launch_bounds__(kBlock) void v3_forward_kernel(const Args<R> a) {
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int groups = a.groups, sub = C / groups;
+  const int64_t total = a.voxels();
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * kBlock) {
+    const Voxel<R> v = locate(a, i);
+    const R *ref_px = a.ref + v.pix * C;
+    R acc = REDUCE == 0 ? R(0) : Limits<R>::min_positive();
+    int used = 0, wn = -1, wgi = -1, wgs = -1;
+    for (int n = 0; n < N; ++n) {
+      Sample<R> s;
+      const int64_t cam = (int64_t)v.b * N + n;
+      project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+      if (s.state != 2) continue;
+      const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
+      int gi = -1, gs = -1;
+      if (REDUCE == 0) {
+        acc += best_pair<R, SUB>(s, t, ref_px, groups, sub, Limits<R>::min_positive(), gi, gs);
+        ++used;
+      } else {
+        const R best = best_pair<R, SUB>(s, t, ref_px, groups, sub, acc, gi, gs);
+        if (gi >= 0) {
+          acc = best;
+          wn = n, wgi = gi, wgs = gs;
+        }
+      }
+    }
+    if (REDUCE == 0) {
+      a.mask[i] = used;
+      a.cost[i] = used > 0 ? acc / static_cast<R>(used) : R(0);
+    } else {
+      a.mask[i * 3] = wn, a.mask[i * 3 + 1] = wgi, a.mask[i * 3 + 2] = wgs;
+      a.cost[i] = wn >= 0 ? acc : R(0);
+    }
+  }
+}
+
+// The D voxels of a pixel all add into the same ref_grad row and the same base-plane
+// gradient.  A workgroup covers kBlock consecutive voxels, i.e. a few consecutive pixels:
+// their rows are accumulated in LDS (ds_add) and leave as one global atomic per element and
+// workgroup.  LDS_ROWS = 0 selects plain global atomics (pixel rows that do not fit).
+template <typename R, int REDUCE, int SUB>
+__global__ __launch_bounds__(kBlock) void v3_backward_kernel(const Args<R> a, int lds_rows) {
+  extern __shared__ __align__(16) unsigned char v3_smem[];
+  R *rows = reinterpret_cast<R *>(v3_smem);  // [lds_rows][C + 1]: ref_grad row, depth gradient
+  const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW, D = (int)a.D;
+  const int groups = a.groups, sub = C / groups;
+  const int64_t total = a.voxels();
+  const int64_t row_step = (int64_t)srcW * C;
+  const int RW = C + 1;
+  // every thread of a workgroup makes the same number of trips: the loop holds barriers
+  for (int64_t base = (int64_t)blockIdx.x * kBlock; base < total;
+       base += (int64_t)gridDim.x * kBlock) {
+    const int64_t pix0 = base / D;
+    if (lds_rows > 0) {
+      for (int k = threadIdx.x; k < lds_rows * RW; k += kBlock) rows[k] = R(0);
+      __syncthreads();
+    }
+    const int64_t i = base + threadIdx.x;
+    const int32_t *m = a.mask_in + (REDUCE == 0 ? i : i * 3);
+    const int32_t m0 = i < total ? m[0] : -1;
+    if (i < total && (REDUCE == 0 ? (m0 > 0) : (m0 >= 0))) {
+      const Voxel<R> v = locate(a, i);
+      const R *ref_px = a.ref + v.pix * C;
+      R *ref_lds = rows + (v.pix - pix0) * RW;  // (kept apart from the global row, so that
+      R *ref_glb = a.ref_grad + v.pix * C;      //  the LDS adds compile to LDS instructions)
+      // :426 cost_grad / (T)mask for the mean; the MIN gradient takes cost_grad as is (:621)
+      const R cg = REDUCE == 0 ? a.cost_grad[i] / static_cast<R>(m0) : a.cost_grad[i];
+      R depth_grad = R(0);
+      const int n_lo = REDUCE == 0 ? 0 : m0, n_hi = REDUCE == 0 ? N : m0 + 1;
+      for (int n = n_lo; n < n_hi && n < N; ++n) {
+        Sample<R> s;
+        const int64_t cam = (int64_t)v.b * N + n;
+        project(a.Rs + cam * 9, a.Ts + cam * 3, v.ref_w, v.ref_h, v.depth, a.half, srcH, srcW, s);
+        // A winner that is not accepted any more (inputs changed since the forward pass) is
+        // skipped; the reference would read and write out of bounds (:593-595).
+        if (s.state != 2) continue;
+        const Taps<R> t = taps_of(a.src, s, cam, C, srcH, srcW);
+        int gi = -1, gs = -1;
+        if (REDUCE == 0) {
+          best_pair<R, SUB>(s, t, ref_px, groups, sub, Limits<R>::min_positive(), gi, gs);
+          // no pair above the seed: the reference indexes group -1 here (:495-496)
+          if (gi < 0) continue;
+        } else {
+          gi = m[1], gs = m[2];
+          if (gi < 0 || gi >= groups || gs < 0 || gs >= groups) continue;
+        }
+        R *g00 = a.src_grad + (t.t00 - a.src);
+        R h_grad = R(0), w_grad = R(0);
+        for (int k = 0; k < sub; ++k) {
+          const int rc = gi * sub + k, cc = gs * sub + k;
+          const R v00 = t.t00[cc], v01 = t.t01[cc], v11 = t.t11[cc], v10 = t.t10[cc];
+          const R smp = s.k00 * v00 + s.k01 * v01 + s.k11 * v11 + s.k10 * v10;
+          if (lds_rows > 0)
+            __hip_atomic_fetch_add(ref_lds + rc, cg * smp, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);
+          else
+            atomic_add(ref_glb + rc, cg * smp);
+          const R bg = cg * ref_px[rc];
+          atomic_add(g00 + cc, bg * s.k00);
+          atomic_add(g00 + C + cc, bg * s.k01);
+          atomic_add(g00 + C + row_step + cc, bg * s.k11);
+          atomic_add(g00 + row_step + cc, bg * s.k10);
+          const R t1 = v11 - v10 - v01 + v00;
+          h_grad += bg * (t1 * s.dw + v10 - v00);
+          w_grad += bg * (t1 * s.dh + v01 - v00);
+        }
+        depth_grad += depth_chain(s, h_grad, w_grad);
+      }
+      if (lds_rows > 0)
+        __hip_atomic_fetch_add(ref_lds + C, depth_grad, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+      else
+        atomic_add(a.depth_grad + v.pix, depth_grad);
+    }
+    if (lds_rows > 0) {
+      __syncthreads();
+      const int64_t pixels = a.pixels();
+      for (int k = threadIdx.x; k < lds_rows * RW; k += kBlock) {
+        const int r = k / RW, c = k - r * RW;
+        const R val = rows[k];
+        if (val != R(0) && pix0 + r < pixels) {
+          if (c < C)
+            atomic_add(a.ref_grad + (pix0 + r) * C + c, val);
+          else
+            atomic_add(a.depth_grad + pix0 + r, val);
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// ---- FeatureAggregate --------------------------------------------------------------------
 template <typename R, int VEC>
 __global__ __launch_bounds__(kBlock) void feature_forward_kernel(const Args<R> a) {
   const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
@@ -275,15 +339,29 @@ bool aligned16(const void *p) {
 
 }  // namespace
 
+// 4 or 8 when a channel group is that many floats and every row starts 16-byte aligned
+// (the pair search then uses 16-byte loads), 0 otherwise.
+template <typename S>
+int v3_vector_width(const Args<S> &a) {
+  const int64_t sub = a.C / a.groups;
+  if (!std::is_same<S, float>::value || (sub != 4 && sub != 8)) return 0;
+  if (!aligned16<S>(a.src) || !aligned16<S>(a.ref)) return 0;
+  return (int)sub;
+}
+
 template <typename S>
 hipError_t launch_v3_forward(const Args<S> &a, hipStream_t stream) {
   const int64_t total = a.voxels();
   if (total == 0) return hipSuccess;
   const int grid = grid_for(total, kBlock);
-  if (a.reduce == 0)
-    v3_forward_kernel<S, 0><<<grid, kBlock, 0, stream>>>(a);
-  else
-    v3_forward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  const int sub = v3_vector_width(a);
+#define CHOP_V3_FWD(RED, SUB) v3_forward_kernel<S, RED, SUB><<<grid, kBlock, 0, stream>>>(a)
+  if (a.reduce == 0) {
+    if (sub == 8) CHOP_V3_FWD(0, 8); else if (sub == 4) CHOP_V3_FWD(0, 4); else CHOP_V3_FWD(0, 0);
+  } else {
+    if (sub == 8) CHOP_V3_FWD(1, 8); else if (sub == 4) CHOP_V3_FWD(1, 4); else CHOP_V3_FWD(1, 0);
+  }
+#undef CHOP_V3_FWD
   return hipGetLastError();
 }
 
@@ -300,10 +378,19 @@ hipError_t launch_v3_backward(const Args<S> &a, hipStream_t stream) {
   const int64_t total = a.voxels();
   if (total == 0 || a.C == 0) return hipSuccess;
   const int grid = grid_for(total, kBlock);
-  if (a.reduce == 0)
-    v3_backward_kernel<S, 0><<<grid, kBlock, 0, stream>>>(a);
-  else
-    v3_backward_kernel<S, 1><<<grid, kBlock, 0, stream>>>(a);
+  const int sub = v3_vector_width(a);
+  // pixels a workgroup's kBlock consecutive voxels can touch, and their rows in LDS
+  int lds_rows = (int)((kBlock + a.D - 1) / a.D) + 1;
+  size_t smem = (size_t)lds_rows * (size_t)(a.C + 1) * sizeof(S);
+  if (smem > 32 * 1024) lds_rows = 0, smem = 0;
+#define CHOP_V3_BWD(RED, SUB) \
+  v3_backward_kernel<S, RED, SUB><<<grid, kBlock, smem, stream>>>(a, lds_rows)
+  if (a.reduce == 0) {
+    if (sub == 8) CHOP_V3_BWD(0, 8); else if (sub == 4) CHOP_V3_BWD(0, 4); else CHOP_V3_BWD(0, 0);
+  } else {
+    CHOP_V3_BWD(1, 0);  // the winner comes from the mask: no pair search
+  }
+#undef CHOP_V3_BWD
   return hipGetLastError();
 }
 
