@@ -964,17 +964,16 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
   ox = nx;
 }
 
-// Adds the four tap images of a finished run into the window; a cell that sticks out of the
-// window goes to memory.  Called from divergent code by all LPP lanes of every pixel whose
-// run just ended.  Float LDS atomics cost several cycles per lane, so for wide pixels
+// Adds the four tap images of a finished run into the window (a cell that sticks out of the
+// window never gets here: flush_cells_to_memory takes it).  Called from divergent code by all
+// LPP lanes of every pixel whose run just ended.  Float LDS atomics cost several cycles per lane, so for wide pixels
 // (LPP >= 4) the window sums are updated with plain 16-byte read-add-write.  Cells of
 // different pixels overlap (a texel is tap 01 of one cell and tap 00 of its neighbour), so
 // the pixels that fire in the same instruction take turns, one pixel per round; usually one
 // or two fire.  Narrow pixels (LPP <= 2: up to 64 pixels per wave) use the atomics instead.
 template <int VEC, int LPP>
 __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4][VEC],
-                                           float *data, float *gview, int srcW, int lane,
-                                           int cl) {
+                                           float *data, int lane, int cl) {
   using WN = Window<VEC, LPP>;
   typedef float vecf __attribute__((ext_vector_type(VEC)));
   if (key < 0) {
@@ -1430,8 +1429,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
               load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + e1), tap[n][3]);
               if (cur[n] >= 0)
                 window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
-                                     s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
-                                     t.lane, t.cl);
+                                     s_data + n * WN::SLOTS * WN::STRIDE, t.lane, t.cl);
               cur[n] = off;
               if constexpr (LPP > 1)
                 cell[n] = lds_at<int2>(smem, p4 * 2u, kCell + ((n * LPP + jj) * PPW) * 8);
@@ -1511,7 +1509,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
                                       t.cl);
     if (cur[n] >= 0 && !out)
       window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
-                           s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW, t.lane, t.cl);
+                           s_data + n * WN::SLOTS * WN::STRIDE, t.lane, t.cl);
   }
   wave_sync();
 #pragma unroll

@@ -441,6 +441,47 @@ def test_large_batch_stress_full_size():
         assert float((a2 - 2 * a1).abs().max()) <= 2e-4 * scale
 
 
+# ---- samples that jump far between consecutive depths ------------------------------------------
+@pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
+def test_backward_cells_outside_the_scatter_window(oracle, C):
+    """A sideways camera offset close to the scene: consecutive depth hypotheses land many
+    texels apart, so most cells lie outside the kernel's scatter window and take its direct
+    path to memory.  One case per lanes-per-pixel variant; FeatureAggregate's gradient runs
+    the same kernel."""
+    rng, geo = np.random.default_rng(C), np.random.default_rng(4)   # one geometry for all widths
+    B, N, H, W, D = 1, 2, 12, 72, 14
+    t = dict(base_plane=geo.uniform(1.0, 1.2, (B, H, W, 1)).astype(np.float32),
+             offsets=geo.permutation(np.linspace(0.0, 3.0, D)).astype(np.float32)[None].repeat(B, 0),
+             ref=rng.normal(size=(B, H, W, C)).astype(np.float32),
+             src=rng.normal(size=(B, N, H, W, C)).astype(np.float32),
+             Rs=np.tile(np.eye(3, dtype=np.float32)[None, None], (B, N, 1, 1)),
+             Ts=np.array([[[40.0, 3.0, 0.0], [-35.0, -2.0, 0.0]]], np.float32).repeat(B, 0))
+    args = tuple(t[k] for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts"))
+    sw, sh, fh, fw, state = oracle.sample_coords(t["base_plane"], t["offsets"], t["Rs"], t["Ts"], (H, W))
+    ok = state == 2
+    jump = np.abs(np.diff(np.where(ok, fw, 0), axis=3))[ok[:, :, :, 1:] & ok[:, :, :, :-1]]
+    assert ok.mean() > 0.2 and np.median(jump) >= 6 and jump.max() > 20   # a chunk spans far more than the 16 texel columns of a window
+    want_cost, want_mask = oracle.cost_volume_fwd(*args)
+    cost, mask = chop.cost_volume_raw(*_v1_inputs(t))
+    _assert_family(0)
+    assert np.array_equal(host(mask), want_mask)
+    assert_forward_close(host(cost), want_cost)
+    cg = rng.standard_normal(want_cost.shape).astype(np.float32)
+    want = oracle.cost_volume_bwd(*args, cg, want_mask)
+    got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), mask)
+    _assert_family(0)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+    fkeys = ("src", "base_plane", "offsets", "Rs", "Ts")
+    _, fmask = oracle.feature_aggregate_fwd(*[t[k] for k in fkeys])
+    fg = rng.standard_normal(fmask.shape[:-1] + (C,)).astype(np.float32)
+    want = oracle.feature_aggregate_bwd(*[t[k] for k in fkeys], fg, fmask)
+    got = chop.feature_aggregate_grad(*[dev(t[k]) for k in fkeys], dev(fg), dev(fmask))
+    _assert_family(0)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+
+
 # ---- every lanes-per-pixel variant of the tiled kernels -------------------------------------
 @pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
 @pytest.mark.parametrize("N", [1, 3])
