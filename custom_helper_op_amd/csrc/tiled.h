@@ -1552,6 +1552,9 @@ inline int choose_segments(int64_t tiles, int64_t D, int lpp, int64_t target_uni
   int nseg = 1;
   const int64_t min_len = lpp > 16 ? lpp : 16;
   while (nseg < 8 && tiles * nseg < target_units && D / (nseg * 2) >= min_len) nseg *= 2;
+  // a problem that does not even give every SIMD one wave: shorter segments still
+  const int64_t short_len = lpp > 4 ? lpp : 4;
+  while (nseg < 16 && tiles * nseg < 1024 && D / (nseg * 2) >= short_len) nseg *= 2;
   return nseg;
 }
 
