@@ -441,6 +441,41 @@ def test_large_batch_stress_full_size():
         assert float((a2 - 2 * a1).abs().max()) <= 2e-4 * scale
 
 
+# ---- five views: the six-view instantiation with one view missing ----------------------------
+@pytest.mark.parametrize("C", [8, 16, 32])
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+def test_five_views(oracle, C, reduce):
+    B, N, H, W, D = 1, 5, 14, 18, 11
+    t = reference_test_case(3, B, N, H, W, C, D, np.float32, seed=C)
+    t["Ts"] = t["Ts"] + np.linspace(-2, 2, N, dtype=np.float32)[None, :, None]   # five different views
+    args = tuple(t[k] for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts"))
+    want_cost, want_mask = oracle.cost_volume_fwd(*args, reduce)
+    cost, mask = chop.cost_volume_raw(*_v1_inputs(t), reduce)
+    _assert_family(0)
+    assert np.array_equal(host(mask), want_mask)
+    if reduce == "MIN":
+        assert np.array_equal(host(cost), want_cost)
+    else:
+        assert_forward_close(host(cost), want_cost)
+    cg = np.random.default_rng(C).standard_normal(want_cost.shape).astype(np.float32)
+    want = oracle.cost_volume_bwd(*args, cg, want_mask, reduce)
+    got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), mask, reduce)
+    _assert_family(0)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+    groups = C // 4
+    depth_grid = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(np.float32)
+    a2 = (t["ref"], t["src"], depth_grid, t["Rs"], t["Ts"])
+    want_cost, want_mask = oracle.cost_volume_v2_fwd(*a2, reduce, groups)
+    cost, mask = chop.cost_volume_v2_raw(*[dev(x) for x in a2], reduce, groups)
+    _assert_family(0)
+    assert np.array_equal(host(mask), want_mask)
+    if reduce == "MIN":
+        assert np.array_equal(host(cost), want_cost)
+    else:
+        assert_forward_close(host(cost), want_cost, atol=1e-5)
+
+
 # ---- samples that jump far between consecutive depths ------------------------------------------
 @pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
 def test_backward_cells_outside_the_scatter_window(oracle, C):
