@@ -12,7 +12,9 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libchop_costvol.so")
-SOURCES = ["api.hip", "general.hip", "v3_feature.hip", "epilogue.hip", "tiled.hip", "tiled_f32.hip", "tiled_f16.hip", "tiled_bf16.hip"]
+SOURCES = ["tiled_f32_fwd.hip", "tiled_f32_bwd.hip", "tiled_f16_fwd.hip", "tiled_f16_bwd.hip",
+           "tiled_bf16_fwd.hip", "tiled_bf16_bwd.hip", "api.hip", "general.hip", "v3_feature.hip",
+           "epilogue.hip", "tiled.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off", "-fno-fast-math",
