@@ -600,3 +600,56 @@ def test_tiled_channel_widths(oracle, C, N):
         _assert_family(0)
         for g, w in zip(got, want):
             assert_backward_close(host(g), w)
+
+
+# ---- HIP graph capture ----------------------------------------------------------------------
+def test_entry_points_replay_in_a_hip_graph(oracle):
+    """The entry points only enqueue kernels (their zero fills are kernels too), so a caller
+    may capture them.  One graph holds a forward and a backward call; it is replayed several
+    times on changing inputs, with eager work and synchronisations in between, and every
+    replay is checked against the oracle."""
+    lib = _lib.load()
+    B, N, H, W, C, D = 1, 2, 16, 20, 32, 24
+    t = reference_test_case(3, B, N, H, W, C, D, np.float32, seed=77)
+    keys = ("ref", "src", "base_plane", "offsets", "Rs", "Ts")
+    ins = {k: dev(t[k]) for k in keys}
+    cost = torch.empty((B, H, W, D, C), device="cuda")
+    mask = torch.empty((B, H, W, D, 1), dtype=torch.int32, device="cuda")
+    cg = torch.empty_like(cost)
+    grads = [torch.empty_like(ins["ref"]), torch.empty_like(ins["src"]), torch.empty_like(ins["base_plane"])]
+    dims = (B, H, W, C, D, N, H, W)
+
+    def step():
+        s = torch.cuda.current_stream().cuda_stream
+        p = [ins[k].data_ptr() for k in keys]
+        assert lib.chop_cost_volume_fwd_f32(s, 0, 1, *dims, *p, cost.data_ptr(), mask.data_ptr()) == 0
+        assert lib.chop_cost_volume_bwd_f32(s, 0, 1, *dims, *p, cg.data_ptr(), mask.data_ptr(),
+                                            *[g.data_ptr() for g in grads]) == 0
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        step()
+    rng = np.random.default_rng(5)
+    for replay in range(4):
+        new_ref = rng.uniform(0, 10, t["ref"].shape).astype(np.float32)
+        new_cg = rng.standard_normal(cost.shape).astype(np.float32)
+        ins["ref"].copy_(dev(new_ref))          # eager work between the replays
+        cg.copy_(dev(new_cg))
+        for g in grads:
+            g.fill_(float("nan"))               # the graph has to zero what it accumulates into
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        args = (new_ref,) + tuple(t[k] for k in keys[1:])
+        want_cost, want_mask = oracle.cost_volume_fwd(*args)
+        want = oracle.cost_volume_bwd(*args, new_cg, want_mask)
+        assert np.array_equal(host(mask), want_mask), replay
+        assert_forward_close(host(cost), want_cost)
+        for g, w in zip(grads, want):
+            assert_backward_close(host(g), w)
