@@ -215,6 +215,11 @@ def main():
                     help="time CostVolumeV3 with this many channel groups on the workload's tensors")
     ap.add_argument("--feature", action="store_true",
                     help="time FeatureAggregate on the workload's tensors")
+    ap.add_argument("--flush-l2", action="store_true",
+                    help="overwrite a 1 GiB scratch buffer before every forward and every backward "
+                         "call, so that L2 and the memory-side cache hold nothing of the workload "
+                         "(the per-call event times then are cold-cache times; value and "
+                         "ms_per_step include the flushes and are not comparable)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
@@ -252,19 +257,25 @@ def main():
         torch.cuda.synchronize()
         del src_buf, dst_buf
     marks = []
+    scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0") if a.flush_l2 else None
     t0 = time.perf_counter()
     for _ in range(a.steps):
-        e0, e1, e2 = ev(), ev(), ev()
+        e0, e1, e2, e3 = ev(), ev(), ev(), ev()
+        if scratch is not None:
+            scratch.fill_(1.0)
         e0.record()
         r.forward()
         e1.record()
-        r.backward()
+        if scratch is not None:
+            scratch.fill_(2.0)
         e2.record()
-        marks.append((e0, e1, e2))
+        r.backward()
+        e3.record()
+        marks.append((e0, e1, e2, e3))
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     fwd_ms = sum(m[0].elapsed_time(m[1]) for m in marks) / len(marks)
-    bwd_ms = sum(m[1].elapsed_time(m[2]) for m in marks) / len(marks)
+    bwd_ms = sum(m[2].elapsed_time(m[3]) for m in marks) / len(marks)
     ms_per_step = wall * 1e3 / a.steps
     fwd_b, bwd_b = wl.algorithmic_bytes()
     dominant = "backward" if bwd_ms >= fwd_ms else "forward"
@@ -289,7 +300,8 @@ def main():
                       "feat": "FeatureAggregate"}[wl.op],
             wl.B, wl.N, wl.H, wl.W,
             wl.C, wl.D, " G%d" % wl.groups if wl.op in ("v2", "v3") else "", wl.storage),
-            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True},
+            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True,
+                   **({"l2_flushed": True} if a.flush_l2 else {})},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": traffic,
