@@ -121,7 +121,7 @@ int backward(void *stream, int reduce, int half_centor, const Dims &d, int group
   if (n_ref == 0 && n_src == 0 && n_depth == 0) return CHOP_OK;
   REQUIRE_PTR(ref_grad, n_ref);
   REQUIRE_PTR(src_grad, n_src);
-  REQUIRE_PTR(depth_grad, n_depth);
+  (void)n_depth;  // depth_grad may be NULL: the depth gradient is then not computed
   const bool work = voxels > 0 && d.C > 0;
   if (work) {
     REQUIRE_PTR(ref, n_ref);

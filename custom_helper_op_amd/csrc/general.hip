@@ -183,7 +183,7 @@ __global__ __launch_bounds__(kBlock) void general_backward_kernel(const Args<S> 
       const R w_grad = g * (t1 * s.dh + v01 - v00);
       depth_grad += depth_chain(s, h_grad, w_grad);
     }
-    atomic_add(a.depth_grad + (a.depth_grid ? i : v.pix), depth_grad);
+    if (a.depth_grad) atomic_add(a.depth_grad + (a.depth_grid ? i : v.pix), depth_grad);
   }
 }
 
@@ -298,7 +298,9 @@ hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream) {
     if ((err = launch_fill_zero(a.ref_grad, (size_t)n_ref * sizeof(S), stream)) != hipSuccess) return err;
     if ((err = launch_fill_zero(a.src_grad, (size_t)n_src * sizeof(S), stream)) != hipSuccess) return err;
   }
-  if ((err = launch_fill_zero(a.depth_grad, (size_t)n_depth * sizeof(R), stream)) != hipSuccess) return err;
+  if (a.depth_grad != nullptr &&
+      (err = launch_fill_zero(a.depth_grad, (size_t)n_depth * sizeof(R), stream)) != hipSuccess)
+    return err;
   const int64_t total = a.voxels() * a.C;
   if (total > 0) {
     const int grid = grid_for(total, kBlock);

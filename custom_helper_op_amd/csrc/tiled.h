@@ -1085,7 +1085,10 @@ constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 :
 // per-channel minimum / per-group maximum (mask = winning view per channel or group; a
 // voxel is skipped when its first entry is negative, cost_volume_kernels_gpu.cu.cc:483-486)
 // and of the summed-squared-difference minimum (mask = the voxel's winning view).
-template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0>
+// DG: false when the caller does not want the depth gradient (a NULL output): the four
+// depth-derivative weights per record and the 20 instructions per wave-iteration that use
+// them drop out.
+template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true>
 __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
   using WN = Window<VEC, LPP>;
@@ -1256,7 +1259,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         float4 dw4 = make_float4(0.f, 0.f, 0.f, 0.f);
         if (t.view0 + n < N && scl != 0.f) {
           reproject<NV>(cam, n, depth, half, g.src_h_max, g.src_w_max, srcW, C, hit);
-          if (hit.off >= 0) {
+          if (DG && hit.off >= 0) {
             // d(sample)/d(depth) = sum over taps of dwt * tap, from
             //   d/d(src_h) = t1*dw + (t10 - t00),  d/d(src_w) = t1*dh + (t01 - t00),
             //   t1 = t11 - t10 - t01 + t00, chained through the perspective divide.
@@ -1298,7 +1301,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           lds_at<int2>(smem, q4 * 2u, kCell + (n * LPP * PPW) * 8) = rec;
           lds_at<float4>(smem, q4 * 4u, kWts + (n * LPP * PPW) * 16) =
               make_float4(hit.k00, hit.k01, hit.k11, hit.k10);
-          lds_at<float4>(smem, q4 * 4u, kDwt + (n * LPP * PPW) * 16) = dw4;
+          if constexpr (DG) lds_at<float4>(smem, q4 * 4u, kDwt + (n * LPP * PPW) * 16) = dw4;
         } else {
           r_off[n] = hit.off;
           r_cell[n] = rec;
@@ -1322,7 +1325,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       if constexpr (LPP > 1) {
         rb_off[0][n] = lds_at<int>(smem, p4, kOff + (n * LPP * PPW) * 4);
         rb_wt[0][n] = lds_at<float4>(smem, p4 * 4u, kWts + (n * LPP * PPW) * 16);
-        rb_dwt[0][n] = lds_at<float4>(smem, p4 * 4u, kDwt + (n * LPP * PPW) * 16);
+        if constexpr (DG)
+          rb_dwt[0][n] = lds_at<float4>(smem, p4 * 4u, kDwt + (n * LPP * PPW) * 16);
+        else
+          rb_dwt[0][n] = make_float4(0.f, 0.f, 0.f, 0.f);
       } else {
         rb_off[0][n] = r_off[n];
         rb_wt[0][n] = r_wts[n];
@@ -1351,7 +1357,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           for (int n = 0; n < NV; ++n) {
             rb_off[nb][n] = lds_at<int>(smem, p4, kOff + ((n * LPP + jj + 1) * PPW) * 4);
             rb_wt[nb][n] = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj + 1) * PPW) * 16);
-            rb_dwt[nb][n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj + 1) * PPW) * 16);
+            if constexpr (DG)
+              rb_dwt[nb][n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj + 1) * PPW) * 16);
+            else
+              rb_dwt[nb][n] = make_float4(0.f, 0.f, 0.f, 0.f);
           }
           rb_scl[nb] = lds_at<float>(smem, p4, kScl + ((jj + 1) * PPW) * 4);
         }
@@ -1460,16 +1469,20 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
               sg[n][1][c] = __builtin_fmaf(gsrc, wt.y, sg[n][1][c]);
               sg[n][2][c] = __builtin_fmaf(gsrc, wt.z, sg[n][2][c]);
               sg[n][3][c] = __builtin_fmaf(gsrc, wt.w, sg[n][3][c]);
-              float ds = dwt.x * tap[n][0][c];
-              ds = __builtin_fmaf(dwt.y, tap[n][1][c], ds);
-              ds = __builtin_fmaf(dwt.z, tap[n][2][c], ds);
-              ds = __builtin_fmaf(dwt.w, tap[n][3][c], ds);
-              dvox = __builtin_fmaf(gsrc, ds, dvox);
+              if constexpr (DG) {
+                float ds = dwt.x * tap[n][0][c];
+                ds = __builtin_fmaf(dwt.y, tap[n][1][c], ds);
+                ds = __builtin_fmaf(dwt.z, tap[n][2][c], ds);
+                ds = __builtin_fmaf(dwt.w, tap[n][3][c], ds);
+                dvox = __builtin_fmaf(gsrc, ds, dvox);
+              }
             }
           }
         }
       }
-      if (per_voxel_depth) {
+      if constexpr (!DG) {
+        // no depth gradient wanted
+      } else if (per_voxel_depth) {
         if constexpr (LPP > 1) {
           const float tot = group_sum<LPP>(dvox);
           if (t.cl == 0) lds_at<float>(smem, p4, kDst + (jj * PPW) * 4) = tot;
@@ -1487,7 +1500,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     }
     if constexpr (LPP > 1) {
       wave_sync();
-      if (per_voxel_depth) {
+      if (DG && per_voxel_depth) {
         const int d = d0 + t.cl;
         if (d < d_hi && t.pix_ok) {
           if (g.ngroups == 1)
@@ -1534,7 +1547,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
     for (int c = 0; c < VEC; ++c) atomic_add(rg + t.pix * C + t.cl * VEC + c, racc[c]);
   }
-  if (!per_voxel_depth) {
+  if (DG && !per_voxel_depth) {
     const float tot = group_sum<LPP>(dacc);
     if (t.cl == 0 && t.pix_ok) {
       if (single)

@@ -122,8 +122,10 @@ def cost_volume_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_m
 
 
 def cost_volume_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_grad, cost_mask,
-                     reduce_method="MEAN", half_centor=True):
-    """The ``CostVolumeGrad`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``."""
+                     reduce_method="MEAN", half_centor=True, need_depth_grad=True):
+    """The ``CostVolumeGrad`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``.
+    With ``need_depth_grad=False`` the third result is ``None`` and the kernels skip the
+    depth-derivative work (the registered op always computes it)."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
@@ -142,7 +144,7 @@ def cost_volume_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_gr
              "cost_mask must have rank 5, and must compate to ref_image")
     ref_grad = torch.empty_like(ref_image)
     src_grad = torch.empty_like(src_images)
-    bp_grad = torch.empty_like(base_plane)
+    bp_grad = torch.empty_like(base_plane) if need_depth_grad else None
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
     if dt in _STORAGE16:
         need = lib.chop_cost_volume_bwd16_workspace_bytes(B, H, W, C, N, *dims[6:])
@@ -190,8 +192,10 @@ def cost_volume_v2_raw(ref_image, src_images, depth_grid, Rs, Ts, reduce_method=
 
 
 def cost_volume_grad_v2(ref_image, src_images, depth_grid, rs, ts, cost_grad, cost_mask,
-                        reduce_method="MEAN", groups=None, half_centor=True):
-    """The ``CostVolumeGradV2`` op: ``(ref_image_grad, src_images_grad, depth_grid_grad)``."""
+                        reduce_method="MEAN", groups=None, half_centor=True,
+                        need_depth_grad=True):
+    """The ``CostVolumeGradV2`` op: ``(ref_image_grad, src_images_grad, depth_grid_grad)``;
+    ``need_depth_grad=False`` as in :func:`cost_volume_grad`."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
@@ -209,7 +213,7 @@ def cost_volume_grad_v2(ref_image, src_images, depth_grid, rs, ts, cost_grad, co
              "cost_mask must have rank 5, and must compate to ref_image")
     ref_grad = torch.empty_like(ref_image)
     src_grad = torch.empty_like(src_images)
-    dg_grad = torch.empty_like(depth_grid)
+    dg_grad = torch.empty_like(depth_grid) if need_depth_grad else None
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
     if dt in _STORAGE16:
         need = lib.chop_cost_volume_bwd16_workspace_bytes(B, H, W, C, N, *dims[6:])
@@ -255,9 +259,10 @@ def cost_aggregate_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduc
 
 
 def cost_aggregate_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_grad, cost_mask,
-                        reduce_method="MEAN", half_centor=True):
+                        reduce_method="MEAN", half_centor=True, need_depth_grad=True):
     """The ``CostAggregateGrad`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``
-    (checks: cost_aggregate_kernels.cc:196-226)."""
+    (checks: cost_aggregate_kernels.cc:196-226); ``need_depth_grad=False`` as in
+    :func:`cost_volume_grad`."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
@@ -276,7 +281,7 @@ def cost_aggregate_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost
              "cost_mask must have rank 4, and must compate to ref_image")
     ref_grad = torch.empty_like(ref_image)
     src_grad = torch.empty_like(src_images)
-    bp_grad = torch.empty_like(base_plane)
+    bp_grad = torch.empty_like(base_plane) if need_depth_grad else None
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
     fn = lib.chop_cost_aggregate_bwd_f32 if dt == torch.float32 else lib.chop_cost_aggregate_bwd_f64
     rc = fn(_stream(ref_grad), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
@@ -438,7 +443,8 @@ class _CostVolume(torch.autograd.Function):
     def backward(ctx, grad_out, _grad_mask):
         ref_image, src_images, base_plane, offsets, Rs, Ts, mask = ctx.saved_tensors
         rg, sg, bg = cost_volume_grad(ref_image, src_images, base_plane, offsets, Rs, Ts,
-                                      grad_out.contiguous(), mask, *ctx.attrs)
+                                      grad_out.contiguous(), mask, *ctx.attrs,
+                                      need_depth_grad=ctx.needs_input_grad[2])
         return rg, sg, bg, None, None, None, None, None
 
 
@@ -458,7 +464,8 @@ class _CostVolumeV2(torch.autograd.Function):
     def backward(ctx, grad_out, _grad_mask):
         ref_image, src_images, depth_grid, Rs, Ts, mask = ctx.saved_tensors
         rg, sg, dg = cost_volume_grad_v2(ref_image, src_images, depth_grid, Rs, Ts,
-                                         grad_out.contiguous(), mask, *ctx.attrs)
+                                         grad_out.contiguous(), mask, *ctx.attrs,
+                                         need_depth_grad=ctx.needs_input_grad[2])
         return rg, sg, dg, None, None, None, None, None
 
 
@@ -478,7 +485,8 @@ class _CostAggregate(torch.autograd.Function):
     def backward(ctx, grad_out, _grad_mask):
         ref_image, src_images, base_plane, offsets, Rs, Ts, mask = ctx.saved_tensors
         rg, sg, bg = cost_aggregate_grad(ref_image, src_images, base_plane, offsets, Rs, Ts,
-                                         grad_out.contiguous(), mask, *ctx.attrs)
+                                         grad_out.contiguous(), mask, *ctx.attrs,
+                                         need_depth_grad=ctx.needs_input_grad[2])
         return rg, sg, bg, None, None, None, None, None
 
 

@@ -75,7 +75,12 @@ int chop_cost_volume_fwd_f64(void *stream, int reduce, int half_centor, int64_t 
  * Replaces functor::CostVolumeGradFunctor<GPUDevice,T,half_centor>::operator()
  * (cost_volume.h:82-133, cost_volume_kernels_gpu.cu.cc:590-655, called from
  * CostVolumeGradOp::Compute, cost_volume_kernels.cc:263-271), including the three
- * SetZeroBig launches (:637-642). */
+ * SetZeroBig launches (:637-642).
+ *
+ * In the CostVolume, CostVolumeV2 and CostAggregate backward entry points the third
+ * gradient (base_plane_grad / depth_grid_grad) may be NULL: it is then neither cleared
+ * nor computed, the other two gradients are unchanged.  The reference always computes
+ * it; a caller whose depth hypotheses are constants saves the work. */
 int chop_cost_volume_bwd_f32(void *stream, int reduce, int half_centor, int64_t B, int64_t H,
                              int64_t W, int64_t C, int64_t D, int64_t N, int64_t srcH,
                              int64_t srcW, const float *ref, const float *src,

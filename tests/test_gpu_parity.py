@@ -301,6 +301,64 @@ def test_autograd_matches_grad_op(oracle):
     assert ins[3].grad is None and ins[4].grad is None and ins[5].grad is None
 
 
+@pytest.mark.parametrize("family", FAMILIES)
+def test_backward_without_the_depth_gradient(oracle, family):
+    """A NULL third gradient: ref_grad and src_grad are those of the full call, the depth
+    gradient is neither written nor computed (V1 both reductions, V2 fp32 and bf16,
+    CostAggregate, and through autograd when the planes do not require a gradient)."""
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(2, hw=(24, 40), depth=24)
+    t = wl.tensors
+    args = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+    for reduce in ("MEAN", "MIN"):
+        _, mask = oracle.cost_volume_fwd(*args, reduce)
+        cg = t["cost_grad"]
+        want = oracle.cost_volume_bwd(*args, cg, mask, reduce)
+        got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), dev(mask), reduce,
+                                    need_depth_grad=False)
+        _assert_family(family)
+        assert got[2] is None
+        assert_backward_close(host(got[0]), want[0])
+        assert_backward_close(host(got[1]), want[1])
+    _, amask = oracle.cost_aggregate_fwd(*args)
+    acg = np.ascontiguousarray(t["cost_grad"][..., 0])
+    want = oracle.cost_aggregate_bwd(*args, acg, amask)
+    got = chop.cost_aggregate_grad(*_v1_inputs(t), dev(acg), dev(amask), need_depth_grad=False)
+    _assert_family(family)
+    assert got[2] is None
+    assert_backward_close(host(got[0]), want[0])
+    assert_backward_close(host(got[1]), want[1])
+
+    wl4 = make_workload(4, hw=(32, 40), batch=1)
+    t4 = wl4.tensors
+    v2 = (t4["ref"], t4["src"], t4["depth_grid"], t4["Rs"], t4["Ts"])
+    _, m4 = oracle.cost_volume_v2_fwd(*v2, "MEAN", 4)
+    want = oracle.cost_volume_v2_bwd(*v2, t4["cost_grad"], m4, "MEAN", 4)
+    ins = [dev(x) for x in v2]
+    got = chop.cost_volume_grad_v2(*ins, dev(t4["cost_grad"]), dev(m4), "MEAN", 4,
+                                   need_depth_grad=False)
+    _assert_family(family)
+    assert got[2] is None
+    assert_backward_close(host(got[0]), want[0])
+    assert_backward_close(host(got[1]), want[1])
+    ins16 = [dev(v2[0], torch.bfloat16), dev(v2[1], torch.bfloat16)] + ins[2:]
+    got = chop.cost_volume_grad_v2(*ins16, dev(t4["cost_grad"], torch.bfloat16), dev(m4),
+                                   "MEAN", 4, need_depth_grad=False)
+    assert got[2] is None
+    _assert_16bit_close(host(got[0]), want[0], "bf16")
+    _assert_16bit_close(host(got[1]), want[1], "bf16")
+
+    ins = _v1_inputs(t)
+    ins[0].requires_grad_(True), ins[1].requires_grad_(True)
+    cost, _ = chop.cost_volume(*ins)
+    (cost * dev(t["cost_grad"])).sum().backward()
+    _, mask = oracle.cost_volume_fwd(*args)
+    want = oracle.cost_volume_bwd(*args, t["cost_grad"], mask)
+    assert_backward_close(host(ins[0].grad), want[0])
+    assert_backward_close(host(ins[1].grad), want[1])
+    assert ins[2].grad is None
+
+
 def test_empty_and_degenerate_inputs():
     z = lambda *s: torch.zeros(*s, device="cuda")
     cost, mask = chop.cost_volume_raw(z(1, 0, 4, 3), z(1, 2, 0, 4, 3), z(1, 0, 4, 1), z(1, 5),
