@@ -212,6 +212,15 @@ int v3_call(void *stream, int reduce, int half_centor, const Dims &d, int groups
   a.cost = cost, a.mask = mask, a.cost_grad = cost_grad, a.mask_in = mask_in;
   a.ref_grad = ref_grad, a.src_grad = src_grad, a.depth_grad = base_plane_grad;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (g_kernel_family == 0 && work) {
+    if constexpr (std::is_same<S, float>::value) {
+      if (backward ? tiled_backward_supported(a) : tiled_forward_supported(a)) {
+        g_last_family = 2;
+        return backward ? launch_status(launch_tiled_backward(a, s), "tiled CostVolumeV3 backward launch")
+                        : launch_status(launch_tiled_forward(a, s), "tiled CostVolumeV3 forward launch");
+      }
+    }
+  }
   g_last_family = 1;
   if (backward) return launch_status(launch_v3_backward(a, s), "CostVolumeV3 backward launch");
   return launch_status(launch_v3_forward(a, s), "CostVolumeV3 forward launch");

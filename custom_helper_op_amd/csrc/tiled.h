@@ -365,6 +365,109 @@ __device__ __forceinline__ void store_ints(int32_t *p, const int *v) {
   }
 }
 
+// ---- CostVolumeV3: the largest correlation of any source group with any reference group ------
+// A value of another lane of the same pixel, in registers.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+// One butterfly step of "largest value, earliest pair on a tie" (both partners end equal).
+template <int CTRL>
+__device__ __forceinline__ void better_pair(float &best, int &code) {
+  const float ob = dpp_move<CTRL>(best);
+  const int oc = dpp_move<CTRL>(code);
+  const bool take = ob > best || (ob == best && oc < code);
+  best = take ? ob : best;
+  code = take ? oc : code;
+}
+constexpr int kNoPair = 0x7fffffff;  // pair code: source group * 16 + reference group
+
+// The best (source group, reference group) pair of one accepted sample of one pixel, found
+// by the pixel's LPP lanes exactly as the reference's loop finds it
+// (cost_volume_kernels_gpu_v3.cu.cc:113-130): lane cl holds the sample of channels
+// 4cl..4cl+3, i.e. part (cl % (SUB/4)) of group cl / (SUB/4); every dot product is one
+// sequential chain over the group's channels, each product and sum rounded separately (for 8
+// channels the even lane's partial sum continues in the odd lane); source group outermost,
+// strict "<" from the smallest positive float, so the earliest pair keeps a tie.
+// `ref_row`: the pixel's reference channels in LDS.  Every lane of the pixel returns the same
+// best value (the seed when no pair exceeds it) and pair code (kNoPair then).
+template <int VEC, int LPP, int SUB>
+__device__ __forceinline__ void v3_best_pair(const float (&smp)[VEC], const float *ref_row, int cl,
+                                             float &best, int &code) {
+  static_assert(VEC == 4 && (SUB == 4 || SUB == 8), "a group is one lane or two");
+  constexpr int C = VEC * LPP, G = C / SUB, LPG = SUB / 4;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const int group = cl / LPG, koff = (cl % LPG) * 4;
+  best = __FLT_MIN__;
+  code = kNoPair;
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    const f4 r = *reinterpret_cast<const f4 *>(ref_row + gi * SUB + koff);
+    const float p0 = smp[0] * r[0], p1 = smp[1] * r[1], p2 = smp[2] * r[2], p3 = smp[3] * r[3];
+    float dot = ((p0 + p1) + p2) + p3;  // (0 + p0 differs from p0 in the sign of zero only)
+    if constexpr (LPG == 2) {
+      const float head = dpp_move<0xA0>(dot);  // quad_perm 0,0,2,2: the even lane's four terms
+      dot = (((head + p0) + p1) + p2) + p3;    // complete in the odd lane
+    }
+    if (best < dot) {
+      best = dot;
+      code = group * 16 + gi;
+    }
+  }
+  if constexpr (LPG == 2) {
+    if ((cl & 1) == 0) best = __FLT_MIN__, code = kNoPair;
+  }
+  if constexpr (LPP >= 2) better_pair<0xB1>(best, code);    // quad_perm 1,0,3,2
+  if constexpr (LPP >= 4) better_pair<0x4E>(best, code);    // quad_perm 2,3,0,1
+  if constexpr (LPP >= 8) better_pair<0x141>(best, code);   // row_half_mirror
+  if constexpr (LPP >= 16) better_pair<0x140>(best, code);  // row_mirror
+}
+
+// The gradient of one accepted sample flows through one pair: the view's best pair, found
+// again as in the forward (REDUCE 0, :469-491), or the recorded winner `pair` (REDUCE 1).
+// Out: gsrc = d(loss)/d(sample) of this lane's channels (zero outside the winning source
+// group); racc += the reference gradient of this lane's channels (zero outside the winning
+// reference group, :494-512).  `rows` = two LDS arrays of 64*VEC floats: the pixel rows of
+// the reference image (written once by the caller) and of this sample.
+template <int VEC, int LPP, int SUB, int REDUCE>
+__device__ __forceinline__ void v3_pair_gradients(const float4 wt, const float (&tap)[4][VEC],
+                                                  float cg, int pair, float *rows, int p, int cl,
+                                                  float (&racc)[VEC], float (&gsrc)[VEC]) {
+  constexpr int C = VEC * LPP, LPG = SUB / 4;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  float *ref_row = rows + p * C, *smp_row = rows + 64 * VEC + p * C;
+  const int group = cl / LPG, koff = (cl % LPG) * 4;
+  float smp[VEC];
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    smp[c] = wt.x * tap[0][c] + wt.y * tap[1][c] + wt.z * tap[2][c] + wt.w * tap[3][c];
+  *reinterpret_cast<f4 *>(smp_row + cl * 4) = f4{smp[0], smp[1], smp[2], smp[3]};
+  int code = pair;
+  if constexpr (REDUCE == 0) {
+    float best;
+    v3_best_pair<VEC, LPP, SUB>(smp, ref_row, cl, best, code);
+  }
+  const bool any = code != kNoPair;
+  const int gi_w = code & 15, gs_w = code >> 4;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) gsrc[c] = 0.f;
+  if (any && group == gs_w) {
+    const f4 r = *reinterpret_cast<const f4 *>(ref_row + gi_w * SUB + koff);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) gsrc[c] = cg * r[c];
+  }
+  wave_sync();  // the sample row is complete
+  if (any && group == gi_w) {
+    const f4 m = *reinterpret_cast<const f4 *>(smp_row + gs_w * SUB + koff);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) racc[c] = __builtin_fmaf(cg, m[c], racc[c]);
+  }
+}
+
 template <int NV>
 constexpr int forward_lds_words(int lpp) {
   return lpp > 1 ? NV * 64 * 5 : 0;
@@ -403,6 +506,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
   float ref[VEC];
   if constexpr (CORR != 4) {
     load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+    if constexpr (CORR == 3) {
+      // CostVolumeV3: every lane of a pixel reads all of the pixel's reference groups
+      static_assert(CORR != 3 || (LPP > 1 && VEC == 4), "CostVolumeV3: wide pixels");
+      float *s_ref = reinterpret_cast<float *>(smem + NV * 64 * 20);  // behind the records
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) s_ref[t.p * (VEC * LPP) + t.cl * VEC + c] = ref[c];
+      wave_sync();
+    }
   } else {
 #pragma unroll
     for (int c = 0; c < VEC; ++c) ref[c] = 0.f;  // the warp-only op has no reference image
@@ -422,7 +533,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
   // summed over all channels (one value per voxel), 4 the samples themselves, one row per
   // (voxel, view), and a 0/1 mask per (voxel, view)
   // (feature_aggregate_kernels_gpu.cu.cc:33-121)
-  const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
+  // 3: CostVolumeV3, per view the largest correlation of any (source group, reference group)
+  // pair; MEAN averages the views' maxima, MIN keeps the largest with (view, reference group,
+  // source group) as its mask (cost_volume_kernels_gpu_v3.cu.cc:52-146, :148-262)
+  const int OC = CORR == 1 ? a.groups : (CORR == 2 || CORR == 3) ? 1 : C;
   const int gv = VEC / g.sub;  // output values per lane
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
@@ -680,6 +794,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       continue;
     }
     float agg_out = 0.f;
+    int v3_out[3] = {-1, -1, -1};
     // ---- phase 2: channel arithmetic by lane (p, channel slice) ---------------------------
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
@@ -699,6 +814,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         arg[c] = -1;
       }
       int k = 0;
+      float v3_acc = REDUCE == 0 ? 0.f : 1.175494351e-38f;  // :76, :193
+      int v3_view = -1, v3_code = 0;
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
         int off;
@@ -709,6 +826,39 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         } else {
           off = r_off[n];
           wt = r_wts[n];
+        }
+        if constexpr (CORR == 3) {
+          if (off >= 0) {
+            if (off != cur[n]) {
+              cur[n] = off;
+              const S *q = view[n] + off;
+              load_vec<S, VEC, false>(q, tap[n][0]);
+              load_vec<S, VEC, false>(q + C, tap[n][1]);
+              load_vec<S, VEC, false>(q + row_step + C, tap[n][2]);
+              load_vec<S, VEC, false>(q + row_step, tap[n][3]);
+            }
+            float smp[VEC];
+#pragma unroll
+            for (int c = 0; c < VEC; ++c)
+              smp[c] = wt.x * tap[n][0][c] + wt.y * tap[n][1][c] + wt.z * tap[n][2][c] +
+                       wt.w * tap[n][3][c];
+            const float *ref_row =
+                reinterpret_cast<const float *>(smem + NV * 64 * 20) + t.p * (VEC * LPP);
+            float best;
+            int code;
+            if (g.sub == 8)
+              v3_best_pair<VEC, LPP, 8>(smp, ref_row, t.cl, best, code);
+            else
+              v3_best_pair<VEC, LPP, 4>(smp, ref_row, t.cl, best, code);
+            if constexpr (REDUCE == 0) {
+              v3_acc += best;  // the seed when no pair exceeds it (:113-131)
+            } else if (v3_acc < best) {
+              // one running maximum over views and pairs (:231-250)
+              v3_acc = best, v3_view = n, v3_code = code;
+            }
+            ++k;
+          }
+          continue;
         }
         if constexpr (CORR == 4) {
           // the sample in the reference's operand order (bit-identical to the plain
@@ -797,6 +947,20 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         }
       }
       if constexpr (CORR == 4) continue;  // every view's row is already stored
+      if constexpr (CORR == 3) {
+        // the lane whose slice index equals the depth's place in the chunk keeps the voxel
+        if (t.cl == jj) {
+          if constexpr (REDUCE == 0) {
+            agg_out = k > 0 ? v3_acc / static_cast<float>(k) : 0.f;  // :136-141
+          } else {
+            agg_out = v3_view >= 0 ? v3_acc : 0.f;  // :253-257
+            v3_out[0] = v3_view;
+            v3_out[1] = v3_view >= 0 ? (v3_code & 15) : -1;
+            v3_out[2] = v3_view >= 0 ? (v3_code >> 4) : -1;
+          }
+        }
+        continue;
+      }
       if constexpr (REDUCE == 1) {
         if (t.pix_ok) {
           S *out = a.cost + (t.pix * D + d) * OC;
@@ -842,9 +1006,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         }
       }
     }
-    if constexpr (CORR == 2 && LPP > 1) {
+    if constexpr ((CORR == 2 || CORR == 3) && LPP > 1) {
       if (t.pix_ok && d0 + t.cl < d_hi)
         __builtin_nontemporal_store(agg_out, reinterpret_cast<float *>(a.cost) + t.pix * D + d0 + t.cl);
+    }
+    if constexpr (CORR == 3 && REDUCE == 1) {
+      if (t.pix_ok && d0 + t.cl < d_hi) {
+        int32_t *m = a.mask + (t.pix * D + d0 + t.cl) * 3;
+        m[0] = v3_out[0], m[1] = v3_out[1], m[2] = v3_out[2];
+      }
     }
     if constexpr (LPP > 1) wave_sync();
   }
@@ -1110,6 +1280,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
                         : reinterpret_cast<int *>(smem) + (LPP > 1 ? NV * 64 * 11 + 128 : 0);
   float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV>();
   float *s_stage = s_data + NV * WN::SLOTS * WN::STRIDE;
+  float *s_v3 = s_stage + 4 * WN::C;  // CORR 3 only: reference rows, sample rows
+  static_assert(CORR != 3 || (NV == 1 && LPP > 1 && VEC == 4), "CostVolumeV3: one view, wide pixels");
   for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
 
   Cameras<NV> cam;
@@ -1119,6 +1291,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   float ref[VEC];
   if constexpr (CORR != 4) {
     load_vec<S, VEC, false>(a.ref + t.pix * C + t.cl * VEC, ref);
+    if constexpr (CORR == 3) {
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) s_v3[t.p * (VEC * LPP) + t.cl * VEC + c] = ref[c];
+    }
   } else {
     static_assert(CORR != 4 || NV == 1, "the warp-only gradient runs one view per workgroup");
 #pragma unroll
@@ -1161,22 +1337,27 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   // summed over all channels (one upstream gradient per voxel), 4 the warp alone: one
   // upstream-gradient row and one 0/1 mask entry per (voxel, view)
   // (feature_aggregate_kernels_gpu.cu.cc:219-326)
-  const int OC = CORR == 1 ? a.groups : CORR == 2 ? 1 : C;
+  // 3: CostVolumeV3, one upstream gradient per voxel that flows through the best group pair
+  constexpr bool kVoxelGrad = CORR == 2 || CORR == 3;
+  const int OC = CORR == 1 ? a.groups : kVoxelGrad ? 1 : C;
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   // upstream-gradient rows fetched ahead; the MIN reduce stages the mask rows beside them
   constexpr int PFMAX = REDUCE ? 4 : 8;
   constexpr int PF = LPP < PFMAX ? LPP : PFMAX;
-  constexpr bool kMaskRows = REDUCE == 1 && CORR != 2;
+  constexpr bool kMaskRows = REDUCE == 1 && !kVoxelGrad;
+  // mask entries per voxel: the MIN reduce of CostVolumeV3 records (view, reference group,
+  // source group)
+  const int mask_w = kMaskRows ? OC : (CORR == 3 && REDUCE == 1) ? 3 : 1;
   // element steps from one depth to the next in the upstream gradient and in the mask
   const int cg_step = CORR == 4 ? N * C : OC;
-  const int cnt_step = kMaskRows ? OC : CORR == 4 ? N : 1;
+  const int cnt_step = CORR == 4 ? N : mask_w;
   const S *cg_lane =
       CORR == 4 ? a.cost_grad + (t.pix * D * N + t.view0) * C + t.cl * VEC
-                : a.cost_grad + t.pix * D * OC + (CORR == 2 ? 0 : t.cl * (CORR ? gv : VEC));
+                : a.cost_grad + t.pix * D * OC + (kVoxelGrad ? 0 : t.cl * (CORR ? gv : VEC));
   const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
   const int32_t *cnt_src = CORR == 4 ? a.mask_in + t.pix * D * N + t.view0
-                                     : a.mask_in + t.pix * D * (kMaskRows ? OC : 1);
+                                     : a.mask_in + t.pix * D * mask_w;
   const int32_t *mask_lane = cnt_src + t.cl * (CORR ? gv : VEC);  // this lane's part of a mask row
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
     // Depth hypothesis and valid-view count of lane (p, j)'s voxel: requested before the
@@ -1184,11 +1365,23 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     // should wait for these two words only.
     float dv = 1.f, cg_vox = 0.f;
     int cnt = REDUCE ? -1 : 0;  // "nothing to do" for a lane without a voxel
+    int v3_pair = kNoPair;
     if (d0 + t.cl < d_hi) {
       dv = dv_src[d0 + t.cl];
       if (t.pix_ok) cnt = cnt_src[(int64_t)(d0 + t.cl) * cnt_step];
-      if constexpr (CORR == 2)  // the voxel's one upstream gradient rides with its record
+      if constexpr (kVoxelGrad)  // the voxel's one upstream gradient rides with its record
         cg_vox = reinterpret_cast<const float *>(cg_lane)[d0 + t.cl];
+      if constexpr (CORR == 3 && REDUCE == 1) {
+        if (t.pix_ok) {
+          const int64_t m3 = (int64_t)(d0 + t.cl) * 3;
+          const int gi = cnt_src[m3 + 1], gs = cnt_src[m3 + 2];
+          // a recorded group outside the image's groups: the voxel is skipped
+          if ((unsigned)gi < (unsigned)a.groups && (unsigned)gs < (unsigned)a.groups)
+            v3_pair = gs * 16 + gi;
+          else
+            cnt = -1;
+        }
+      }
     }
     int r_off[NV];
     int2 r_cell[NV];
@@ -1199,7 +1392,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     // reprojection below overlaps their latency.  Streaming loads: cached ones let the
     // next view's workgroup hit L2 more often (690 -> 660 MB fetched) and save 10 us here,
     // but leave the caches full of these rows and cost the next forward launch 25 us.
-    float cgr[CORR == 2 ? 1 : PF][VEC];
+    float cgr[kVoxelGrad ? 1 : PF][VEC];
     int mrow[kMaskRows ? PF : 1][VEC];
     auto load_rows = [&](int first) {
 #pragma unroll
@@ -1227,7 +1420,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         }
       }
     };
-    if constexpr (CORR != 2) load_rows(d0);
+    if constexpr (!kVoxelGrad) load_rows(d0);
     {
       const float depth = d0 + t.cl < d_hi ? (per_voxel_depth ? dv : base + dv) : 1.f;
       // factor the reduce applies to the upstream gradient: squared difference 2/k,
@@ -1238,6 +1431,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         if (cnt > 0) {
           if constexpr (CORR == 2)
             scl = 2.f * (cg_vox / static_cast<float>(cnt * C));
+          else if constexpr (CORR == 3)
+            scl = cg_vox / static_cast<float>(cnt);  // cost_volume_kernels_gpu_v3.cu.cc:426
           else
             scl = (CORR == 0 ? 2.f : 1.f) * __builtin_amdgcn_rcpf(static_cast<float>(cnt));
         }
@@ -1246,6 +1441,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         // for the summed squared difference, its winning view)
         if constexpr (CORR == 2) {
           if (cnt == t.view0) scl = 2.f * (cg_vox / static_cast<float>(C));
+        } else if constexpr (CORR == 3) {
+          if (cnt == t.view0) scl = cg_vox;  // cost_volume_kernels_gpu_v3.cu.cc:621-622
         } else {
           if (cnt >= 0) scl = CORR == 0 ? 2.f : 1.f;
         }
@@ -1311,7 +1508,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       }
       if constexpr (LPP > 1) {
         lds_at<float>(smem, q4, kScl) = scl;
-        lds_at<float>(smem, q4, kDst) = 0.f;
+        if constexpr (CORR == 3)
+          lds_at<int>(smem, q4, kDst) = v3_pair;  // (this op has no per-voxel depth gradient)
+        else
+          lds_at<float>(smem, q4, kDst) = 0.f;
       } else {
         r_scl = scl;
       }
@@ -1345,7 +1545,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       if (d >= d_hi) {
         if constexpr (LPP >= 16) continue; else break;  // see the forward kernel
       }
-      if constexpr (LPP > PF && CORR != 2) {
+      if constexpr (LPP > PF && !kVoxelGrad) {
         if (jj > 0 && jj % PF == 0) load_rows(d0 + jj);  // next part of a deep chunk
       }
       // The records of the NEXT depth are requested now, so that their LDS latency overlaps
@@ -1386,8 +1586,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       if (scl != 0.f) {
         float cg[VEC];
         {
-          const float *raw = cgr[CORR == 2 ? 0 : jj % PF];
-          if constexpr (CORR == 2) {
+          const float *raw = cgr[kVoxelGrad ? 0 : jj % PF];
+          if constexpr (kVoxelGrad) {
 #pragma unroll
             for (int c = 0; c < VEC; ++c) cg[c] = scl;
           } else if (CORR == 0 || g.sub == 1) {
@@ -1445,10 +1645,22 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
               else
                 cell[n] = r_cell[n];
             }
+            float gs3[VEC];
+            if constexpr (CORR == 3) {
+              const int pair = REDUCE ? lds_at<int>(smem, p4, kDst + (jj * PPW) * 4) : 0;
+              if (g.sub == 8)
+                v3_pair_gradients<VEC, LPP, 8, REDUCE>(wt, tap[n], scl, pair, s_v3, t.p, t.cl, racc,
+                                                       gs3);
+              else
+                v3_pair_gradients<VEC, LPP, 4, REDUCE>(wt, tap[n], scl, pair, s_v3, t.p, t.cl, racc,
+                                                       gs3);
+            }
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
               float gsrc;  // d(loss)/d(sample of this channel)
-              if constexpr (CORR == 4) {
+              if constexpr (CORR == 3) {
+                gsrc = gs3[c];
+              } else if constexpr (CORR == 4) {
                 gsrc = cg[c];
               } else if (CORR != 1) {
                 float diff = __builtin_fmaf(wt.x, tap[n][0][c], -ref[c]);

@@ -93,6 +93,103 @@ def test_v3_backward(oracle, shape, reduce, dtype):
             assert_backward_close(host(g), w, rtol=1e-4 if dtype == np.float32 else 1e-10)
 
 
+@pytest.mark.parametrize("C,G", [(8, 1), (8, 2), (16, 2), (16, 4), (32, 4), (32, 8), (64, 8),
+                                 (64, 16)])
+@pytest.mark.parametrize("N", [1, 3])
+def test_v3_tiled_widths(oracle, C, G, N):
+    """Groups of 4 and 8 channels (one lane or two per group) at 2, 4, 8 and 16 lanes per
+    pixel run the tiled kernels in float32.  Forward: cost and all indices bit for bit, like
+    the one-thread-per-voxel kernel.  Gradient: within the backward bar, including the best
+    pair it finds again for MEAN."""
+    B, H, W, D = 2, 20, 24, 21
+    lib = _lib.load()
+    rng = np.random.default_rng(C + G + N)
+    for case in (1, 3):
+        t = reference_test_case(case, B, N, H, W, C, D, np.float32, seed=200 + case)
+        for reduce in ("MEAN", "MIN"):
+            want_cost, mask = oracle.cost_volume_v3_fwd(*_args(t), reduce, G)
+            for family in (1, 0):
+                lib.chop_set_kernel_family(family)
+                cost, got_mask = chop.cost_volume_v3_raw(*_inputs(t), reduce, G)
+                assert lib.chop_last_kernel_family() == (2 if family == 0 else 1)
+                assert np.array_equal(host(got_mask), mask)
+                assert np.array_equal(host(cost), want_cost)
+            if reduce == "MIN":
+                # recorded groups outside the image's groups: such voxels are skipped
+                mask = mask.copy()
+                flat = mask.reshape(-1, 3)
+                hit = np.flatnonzero(flat[:, 0] >= 0)
+                flat[hit[::7], 1] = G
+                flat[hit[3::11], 2] = -1
+            cg = rng.normal(size=(B, H, W, D, 1)).astype(np.float32)
+            want = oracle.cost_volume_v3_bwd(*_args(t), cg, mask, reduce, G)
+            for family in (1, 0):
+                lib.chop_set_kernel_family(family)
+                got = chop.cost_volume_grad_v3(*_inputs(t), dev(cg), dev(mask), reduce, G)
+                assert lib.chop_last_kernel_family() == (2 if family == 0 else 1)
+                for g, w in zip(got, want):
+                    assert_backward_close(host(g), w)
+    lib.chop_set_kernel_family(0)
+
+
+@pytest.mark.parametrize("C,G", [(16, 4), (32, 4), (64, 8)])
+def test_v3_tiled_ties(oracle, C, G):
+    """Equal correlations: the first pair in (source group, reference group) order wins, in
+    the lanes' tournament as in the reference's loop.  Constant images make every pair tie;
+    reference groups 1 and 2 doubled make those two tie ahead of the rest."""
+    B, N, H, W, D = 1, 2, 12, 16, 9
+    lib = _lib.load()
+    t = reference_test_case(1, B, N, H, W, C, D, np.float32, seed=5)
+    t["src"] = np.ones_like(t["src"])
+    rng = np.random.default_rng(3)
+    for variant in (0, 1):
+        ref = np.ones_like(t["ref"])
+        if variant == 1:
+            sub = C // G
+            ref[..., sub:3 * sub] = 2.0
+        t["ref"] = ref
+        _, mask = oracle.cost_volume_v3_fwd(*_args(t), "MEAN", G)
+        want_cost, want_win = oracle.cost_volume_v3_fwd(*_args(t), "MIN", G)
+        lib.chop_set_kernel_family(0)
+        cost, win = chop.cost_volume_v3_raw(*_inputs(t), "MIN", G)
+        assert lib.chop_last_kernel_family() == 2
+        assert np.array_equal(host(win), want_win) and np.array_equal(host(cost), want_cost)
+        seen = want_win.reshape(-1, 3)
+        seen = seen[seen[:, 0] >= 0]
+        assert len(seen) and (seen[:, 0] == 0).all() and (seen[:, 2] == 0).all()
+        assert (seen[:, 1] == (0 if variant == 0 else 1)).all()
+        cg = rng.normal(size=(B, H, W, D, 1)).astype(np.float32)
+        want = oracle.cost_volume_v3_bwd(*_args(t), cg, mask, "MEAN", G)
+        # the whole reference gradient sits in the winning group
+        sub = C // G
+        first = slice(0, sub) if variant == 0 else slice(sub, 2 * sub)
+        outside = np.delete(want[0], np.r_[first], axis=-1)
+        assert np.abs(want[0][..., first]).max() > 0 and not outside.any()
+        lib.chop_set_kernel_family(0)
+        got = chop.cost_volume_grad_v3(*_inputs(t), dev(cg), dev(mask), "MEAN", G)
+        assert lib.chop_last_kernel_family() == 2
+        assert_backward_close(host(got[0]), want[0])
+        assert_backward_close(host(got[1]), want[1])
+        # constant images: the depth gradient is exactly zero in the reference's form
+        # (differences of equal taps); the tiled kernel sums four weights that cancel
+        assert not want[2].any() and np.abs(host(got[2])).max() < 1e-6
+
+
+def test_v3_backward_full_size(oracle):
+    """CostVolumeV3's gradient on the benchmark workload's tensors, both reduces."""
+    t = make_workload(2, with_cost_grad=False).tensors
+    ins = _inputs(t)
+    rng = np.random.default_rng(11)
+    cg = rng.normal(size=(1, 128, 160, 192, 1)).astype(np.float32)
+    for reduce in ("MEAN", "MIN"):
+        _, mask = chop.cost_volume_v3_raw(*ins, reduce, 4)
+        got = chop.cost_volume_grad_v3(*ins, dev(cg), mask, reduce, 4)
+        assert _lib.load().chop_last_kernel_family() == 2
+        want = oracle.cost_volume_v3_bwd(*_args(t), cg, host(mask), reduce, 4)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+
+
 def test_v3_autograd_and_errors(oracle):
     t = reference_test_case(3, 2, 2, 8, 10, 6, 4, np.float64, seed=2)
     ins = _inputs(t)
@@ -233,6 +330,7 @@ def test_full_size_benchmark_tensors(oracle):
     ins = _inputs(t)
     for reduce in ("MEAN", "MIN"):
         cost, mask = chop.cost_volume_v3_raw(*ins, reduce, 4)
+        assert _lib.load().chop_last_kernel_family() == 2
         want_cost, want_mask = oracle.cost_volume_v3_fwd(*_args(t), reduce, 4, threads=16)
         assert np.array_equal(host(mask), want_mask)
         assert np.array_equal(host(cost), want_cost)
