@@ -12,7 +12,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libchop_costvol.so")
-SOURCES = ["tiled_f32_fwd.hip", "tiled_f32_bwd.hip", "tiled_f16_fwd.hip", "tiled_f16_bwd.hip",
+SOURCES = ["tiled_f32_fwd_wide.hip", "tiled_f32_bwd_wide.hip", "tiled_f32_fwd_narrow.hip",
+           "tiled_f32_bwd_narrow.hip", "tiled_f16_fwd.hip", "tiled_f16_bwd.hip",
            "tiled_bf16_fwd.hip", "tiled_bf16_bwd.hip", "api.hip", "general.hip", "v3_feature.hip",
            "epilogue.hip", "tiled.hip"]
 FLAGS = [

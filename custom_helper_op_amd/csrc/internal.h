@@ -115,6 +115,12 @@ template <typename S>
 bool tiled_backward_supported(const Args<S> &a);
 template <typename S>
 hipError_t launch_tiled_backward(const Args<S> &a, hipStream_t stream);
+// Between the translation units of one direction and storage type: the kernels for 8 and 16
+// lanes per pixel, where those are compiled apart from the rest.
+template <typename S>
+hipError_t launch_tiled_forward_wide(const Args<S> &a, hipStream_t stream);
+template <typename S>
+hipError_t launch_tiled_backward_wide(const Args<S> &a, hipStream_t stream);
 
 // Utility launches.
 hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);

@@ -1,0 +1,6 @@
+// Tiled cost-volume kernels instantiated for float storage: backward, 1 to 4 lanes per
+// pixel, and the public entry points of this direction.
+#define CHOP_S float
+#define CHOP_TILED_BACKWARD
+#define CHOP_LPP_PART 0
+#include "tiled_launch.inc"
