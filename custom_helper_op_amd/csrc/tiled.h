@@ -1072,8 +1072,10 @@ constexpr int backward_record_words() {
 template <int VEC, int LPP, int NV>
 constexpr int backward_lds_words() {
   using WN = Window<VEC, LPP>;
-  // records (or list), windows, and one cell (4 texels x C) staged on its way to memory
-  return backward_record_words<VEC, LPP, NV>() + NV * WN::SLOTS * WN::STRIDE + 4 * WN::C;
+  // records (or list), windows, one cell (4 texels x C) staged on its way to memory, and for
+  // narrow pixels one claim word per window slot
+  return backward_record_words<VEC, LPP, NV>() + NV * WN::SLOTS * WN::STRIDE + 4 * WN::C +
+         (LPP <= 2 ? WN::SLOTS : 0);
 }
 
 // Minimum over the 64 lanes, in registers: four DPP steps reduce each row of 16 lanes,
@@ -1136,14 +1138,18 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
 
 // Adds the four tap images of a finished run into the window (a cell that sticks out of the
 // window never gets here: flush_cells_to_memory takes it).  Called from divergent code by all
-// LPP lanes of every pixel whose run just ended.  Float LDS atomics cost several cycles per lane, so for wide pixels
-// (LPP >= 4) the window sums are updated with plain 16-byte read-add-write.  Cells of
-// different pixels overlap (a texel is tap 01 of one cell and tap 00 of its neighbour), so
-// the pixels that fire in the same instruction take turns, one pixel per round; usually one
-// or two fire.  Narrow pixels (LPP <= 2: up to 64 pixels per wave) use the atomics instead.
+// LPP lanes of every pixel whose run just ended.  Float LDS atomics cost about three cycles
+// per lane, so the window sums are updated with plain 16-byte read-add-write.  Cells of
+// different pixels overlap (a texel is tap 01 of one cell and tap 00 of its neighbour).
+// Wide pixels (LPP >= 4, at most 16 pixels per wave, usually one or two firing): the pixels
+// that fire in the same instruction take turns, one pixel per round.  Narrow pixels (up to
+// 64 per wave, a dozen firing): all of them add tap 00, then all tap 01, ... — two pixels
+// then collide only if they are on the SAME cell, and those are told apart by a claim: every
+// pending pixel writes its number into the claim word of its first texel's slot and the one
+// that reads its own number back goes ahead; the others try again (`tags`: one word per slot).
 template <int VEC, int LPP>
 __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4][VEC],
-                                           float *data, int lane, int cl) {
+                                           float *data, int *tags, int lane, int cl) {
   using WN = Window<VEC, LPP>;
   typedef float vecf __attribute__((ext_vector_type(VEC)));
   if (key < 0) {
@@ -1180,12 +1186,27 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
         if (firing) wave_sync();
       }
     } else {
+      const int me = lane - cl;  // the same in both lanes of a pixel
+      bool pending = true;
+      while (true) {
+        if (pending) tags[slot[0]] = me;
+        wave_sync();
+        const bool go = pending && tags[slot[0]] == me;
+        if (go) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        float *d = base + slot[k] * WN::STRIDE;
+          for (int k = 0; k < 4; ++k) {
+            vecf *d = reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE);
+            vecf old = *d;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i)
-          __hip_atomic_fetch_add(d + i, v[k][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+            for (int i = 0; i < VEC; ++i) old[i] += v[k][i];
+            *d = old;
+            // (the next tap may be the texel another pixel has just updated: the LDS keeps a
+            // wave's operations in order, the compiler is held to it here)
+            wave_sync();
+          }
+        }
+        pending = pending && !go;
+        if (__ballot(pending) == 0ull) break;
       }
     }
   }
@@ -1280,7 +1301,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
                         : reinterpret_cast<int *>(smem) + (LPP > 1 ? NV * 64 * 11 + 128 : 0);
   float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV>();
   float *s_stage = s_data + NV * WN::SLOTS * WN::STRIDE;
-  float *s_v3 = s_stage + 4 * WN::C;  // CORR 3 only: reference rows, sample rows
+  int *s_tags = reinterpret_cast<int *>(s_stage + 4 * WN::C);  // narrow pixels: claim words
+  static_assert(LPP > 2 || NV == 1, "one set of claim words: one view per workgroup");
+  // CORR 3 only: reference rows, sample rows
+  float *s_v3 = s_stage + 4 * WN::C + (LPP <= 2 ? WN::SLOTS : 0);
   static_assert(CORR != 3 || (NV == 1 && LPP > 1 && VEC == 4), "CostVolumeV3: one view, wide pixels");
   for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
 
@@ -1638,7 +1662,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
               load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + e1), tap[n][3]);
               if (cur[n] >= 0)
                 window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
-                                     s_data + n * WN::SLOTS * WN::STRIDE, t.lane, t.cl);
+                                     s_data + n * WN::SLOTS * WN::STRIDE, s_tags, t.lane, t.cl);
               cur[n] = off;
               if constexpr (LPP > 1)
                 cell[n] = lds_at<int2>(smem, p4 * 2u, kCell + ((n * LPP + jj) * PPW) * 8);
@@ -1734,7 +1758,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
                                       t.cl);
     if (cur[n] >= 0 && !out)
       window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
-                           s_data + n * WN::SLOTS * WN::STRIDE, t.lane, t.cl);
+                           s_data + n * WN::SLOTS * WN::STRIDE, s_tags, t.lane, t.cl);
   }
   wave_sync();
 #pragma unroll
