@@ -539,6 +539,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
   const int OC = CORR == 1 ? a.groups : (CORR == 2 || CORR == 3) ? 1 : C;
   const int gv = VEC / g.sub;  // output values per lane
   const int d_lo = t.d_lo, d_hi = t.d_hi;
+  // this pixel's output rows (the 64-bit product once per wave, not once per depth)
+  S *const out_pix = a.cost + t.pix * D * OC;
+  int32_t *const mask_pix = a.mask + t.pix * D * OC;
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
     // ---- phase 1: reprojection by lane (p, j = cl) --------------------------------------
     int r_off[NV];
@@ -762,9 +765,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       for (int jj = 0; jj < DB; ++jj) {
         const int d = d0 + j0 + jj;
         if (d >= d_hi || !t.pix_ok) continue;
-        S *out = a.cost + (t.pix * D + d) * OC;
+        S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
         if constexpr (REDUCE == 1) {
-          int32_t *mout = a.mask + (t.pix * D + d) * OC;
+          int32_t *mout = mask_pix + d * OC;
           if (CORR == 0) {
             store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
             store_ints<VEC>(mout + t.cl * VEC, arg[jj]);
@@ -963,8 +966,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       }
       if constexpr (REDUCE == 1) {
         if (t.pix_ok) {
-          S *out = a.cost + (t.pix * D + d) * OC;
-          int32_t *mout = a.mask + (t.pix * D + d) * OC;
+          S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
+          int32_t *mout = mask_pix + d * OC;
           if (CORR == 0) {
             store_vec<S, VEC, true>(out + t.cl * VEC, acc);
             store_ints<VEC>(mout + t.cl * VEC, arg);
@@ -996,7 +999,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         for (int c = 0; c < VEC; ++c) acc[c] *= inv;
       }
       if (t.pix_ok) {
-        S *out = a.cost + (t.pix * D + d) * OC;
+        S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
         if (CORR == 0) {
           store_vec<S, VEC, true>(out + t.cl * VEC, acc);
         } else {
