@@ -1124,15 +1124,25 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
     if (count > 0) {
       wave_sync();
       constexpr int EPI = 64 / WN::C;  // texels per instruction
+      constexpr int UN = 4;            // instructions per round: their LDS reads go out together
       const int sub_e = lane / WN::C, j = lane - sub_e * WN::C;
-      for (int e0 = 0; e0 < count; e0 += EPI) {
-        const int e = e0 + sub_e;
-        if (e < count) {
-          float *d = data + list[2 * e] * WN::STRIDE + j;
-          const float v = *d;
-          if (v != 0.f) {
-            *d = 0.f;
-            atomic_add(gview + (int64_t)list[2 * e + 1] * WN::C + j, v);
+      const int2 *pairs = reinterpret_cast<const int2 *>(list);
+      for (int e0 = 0; e0 < count; e0 += UN * EPI) {
+        int2 le[UN];
+        float v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          const int e = e0 + u * EPI + sub_e;
+          le[u] = pairs[e < count ? e : 0];
+          if (e >= count) le[u].x = -1;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) v[u] = le[u].x >= 0 ? data[le[u].x * WN::STRIDE + j] : 0.f;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          if (v[u] != 0.f) {
+            data[le[u].x * WN::STRIDE + j] = 0.f;
+            atomic_add(gview + (int64_t)le[u].y * WN::C + j, v[u]);
           }
         }
       }
@@ -1332,7 +1342,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   // CORR 3 only: reference rows, sample rows
   float *s_v3 = s_stage + 4 * WN::C + (LPP <= kClaimLanes ? WN::SLOTS : 0);
   static_assert(CORR != 3 || (NV == 1 && LPP > 1 && VEC == 4), "CostVolumeV3: one view, wide pixels");
-  for (int k = t.lane; k < NV * WN::SLOTS * WN::STRIDE; k += 64) s_data[k] = 0.f;
+  for (int k = t.lane * 4; k < NV * WN::SLOTS * WN::STRIDE; k += 256)
+    *reinterpret_cast<float4 *>(s_data + k) = make_float4(0.f, 0.f, 0.f, 0.f);
 
   Cameras<NV> cam;
   load_cameras<S, NV>(a, t.b, t.view0, static_cast<float>(t.w) + half,
