@@ -663,9 +663,10 @@ def test_tiled_channel_widths(oracle, C, N):
 # ---- HIP graph capture ----------------------------------------------------------------------
 def test_entry_points_replay_in_a_hip_graph(oracle):
     """The entry points only enqueue kernels (their zero fills are kernels too), so a caller
-    may capture them.  One graph holds a forward and a backward call; it is replayed several
-    times on changing inputs, with eager work and synchronisations in between, and every
-    replay is checked against the oracle."""
+    may capture them.  One graph holds a CostVolume forward and backward call, a backward call
+    without the depth gradient and a CostVolumeV3 forward and backward call; it is replayed
+    several times on changing inputs, with eager work and synchronisations in between, and
+    every replay is checked against the oracle."""
     lib = _lib.load()
     B, N, H, W, C, D = 1, 2, 16, 20, 32, 24
     t = reference_test_case(3, B, N, H, W, C, D, np.float32, seed=77)
@@ -675,6 +676,11 @@ def test_entry_points_replay_in_a_hip_graph(oracle):
     mask = torch.empty((B, H, W, D, 1), dtype=torch.int32, device="cuda")
     cg = torch.empty_like(cost)
     grads = [torch.empty_like(ins["ref"]), torch.empty_like(ins["src"]), torch.empty_like(ins["base_plane"])]
+    grads2 = [torch.empty_like(ins["ref"]), torch.empty_like(ins["src"])]
+    cost3 = torch.empty((B, H, W, D, 1), device="cuda")
+    mask3 = torch.empty((B, H, W, D, 1), dtype=torch.int32, device="cuda")
+    cg3 = torch.empty_like(cost3)
+    grads3 = [torch.empty_like(g) for g in grads]
     dims = (B, H, W, C, D, N, H, W)
 
     def step():
@@ -683,6 +689,14 @@ def test_entry_points_replay_in_a_hip_graph(oracle):
         assert lib.chop_cost_volume_fwd_f32(s, 0, 1, *dims, *p, cost.data_ptr(), mask.data_ptr()) == 0
         assert lib.chop_cost_volume_bwd_f32(s, 0, 1, *dims, *p, cg.data_ptr(), mask.data_ptr(),
                                             *[g.data_ptr() for g in grads]) == 0
+        assert lib.chop_cost_volume_bwd_f32(s, 0, 1, *dims, *p, cg.data_ptr(), mask.data_ptr(),
+                                            *[g.data_ptr() for g in grads2], None) == 0
+        assert lib.chop_cost_volume_v3_fwd_f32(s, 0, 1, *dims, 4, *p, cost3.data_ptr(),
+                                               mask3.data_ptr()) == 0
+        assert lib.chop_last_kernel_family() == 2
+        assert lib.chop_cost_volume_v3_bwd_f32(s, 0, 1, *dims, 4, *p, cg3.data_ptr(),
+                                               mask3.data_ptr(), *[g.data_ptr() for g in grads3]) == 0
+        assert lib.chop_last_kernel_family() == 2
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -699,7 +713,9 @@ def test_entry_points_replay_in_a_hip_graph(oracle):
         new_cg = rng.standard_normal(cost.shape).astype(np.float32)
         ins["ref"].copy_(dev(new_ref))          # eager work between the replays
         cg.copy_(dev(new_cg))
-        for g in grads:
+        new_cg3 = rng.standard_normal(cost3.shape).astype(np.float32)
+        cg3.copy_(dev(new_cg3))
+        for g in grads + grads2 + grads3:
             g.fill_(float("nan"))               # the graph has to zero what it accumulates into
         torch.cuda.synchronize()
         graph.replay()
@@ -710,4 +726,10 @@ def test_entry_points_replay_in_a_hip_graph(oracle):
         assert np.array_equal(host(mask), want_mask), replay
         assert_forward_close(host(cost), want_cost)
         for g, w in zip(grads, want):
+            assert_backward_close(host(g), w)
+        for g, w in zip(grads2, want[:2]):
+            assert_backward_close(host(g), w)
+        want_cost3, want_mask3 = oracle.cost_volume_v3_fwd(*args, "MEAN", 4)
+        assert np.array_equal(host(mask3), want_mask3) and np.array_equal(host(cost3), want_cost3)
+        for g, w in zip(grads3, oracle.cost_volume_v3_bwd(*args, new_cg3, want_mask3, "MEAN", 4)):
             assert_backward_close(host(g), w)
