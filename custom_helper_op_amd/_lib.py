@@ -37,6 +37,8 @@ for _t in ("f32", "f64"):
     SIGNATURES["chop_cost_volume_sample_coords_" + _t] = [_vp, _int] + [_i64] * 7 + [_vp] * 10
 SIGNATURES["chop_cost_volume_fwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 9
 SIGNATURES["chop_cost_volume_bwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 13 + [ctypes.c_size_t]
+SIGNATURES["chop_cost_volume_bwd_16_static"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 12
+SIGNATURES["chop_static_scratch_bytes"] = []
 SIGNATURES["chop_cost_volume_v2_fwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 7
 SIGNATURES["chop_cost_volume_v2_bwd_16"] = ([_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 11
                                             + [ctypes.c_size_t])
@@ -66,6 +68,7 @@ def load():
         fn.restype = _int
     lib.chop_last_error_string.restype = ctypes.c_char_p
     lib.chop_cost_volume_bwd16_workspace_bytes.restype = ctypes.c_size_t
+    lib.chop_static_scratch_bytes.restype = ctypes.c_size_t
     _lib = lib
     return lib
 

@@ -3,6 +3,7 @@
 // (custom_helper_op/cc/kernels/cost_volume_kernels.cc:91-106, :220-243 and
 // cost_volume_kernels_v2.cc:93-110) as far as they can be expressed on raw pointers and
 // sizes; it runs before any HIP call, so bad arguments are reported on any machine.
+#include <atomic>
 #include <cstdio>
 #include <limits>
 #include <string>
@@ -277,6 +278,37 @@ int feature_call(void *stream, int half_centor, const Dims &d, const S *src, con
   g_last_family = 1;
   if (backward) return launch_status(launch_feature_backward(a, s), "FeatureAggregate backward launch");
   return launch_status(launch_feature_forward(a, s), "FeatureAggregate forward launch");
+}
+
+// ---- scratch of the entry point that allocates nothing ---------------------------------------
+// chop_cost_volume_bwd_16_static keeps the fp32 gradient images of the 16-bit backward in
+// this array instead of a caller-supplied workspace.  Every GPU the library runs on holds its
+// own copy of the array (at its own address) from the moment the code object is loaded until
+// the process ends.  On the host the name `scratch` is only a handle for hipGetSymbolAddress;
+// kernels, fills and copies get the per-device address that call returns.
+constexpr size_t kScratchBytes = (size_t)32 << 20;  // 32 MiB per GPU
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Address of `scratch` on the current device; looked up once per device (a race between two
+// first calls stores the same address twice).  Returns nullptr with *err set on failure.
+void *scratch_on_current_device(hipError_t *err) {
+  int dev = -1;
+  *err = hipGetDevice(&dev);
+  if (*err != hipSuccess) return nullptr;
+  if (dev < 0 || dev >= kMaxDevices) {
+    *err = hipErrorInvalidDevice;
+    return nullptr;
+  }
+  void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    *err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (*err != hipSuccess) return nullptr;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  return p;
 }
 
 }  // namespace
@@ -570,6 +602,36 @@ int chop_cost_volume_bwd_16(void *stream, int storage, int reduce, int half_cent
                        (const bf16_t *)ref, (const bf16_t *)src, base_plane, offsets, depth_grid,
                        Rs, Ts, (const bf16_t *)cost_grad, mask, (bf16_t *)ref_grad,
                        (bf16_t *)src_grad, depth_grad, false, workspace, workspace_bytes))
+}
+
+size_t chop_static_scratch_bytes(void) { return kScratchBytes; }
+
+int chop_cost_volume_bwd_16_static(void *stream, int storage, int reduce, int half_centor,
+                                   int64_t B, int64_t H, int64_t W, int64_t C, int64_t D,
+                                   int64_t N, int64_t srcH, int64_t srcW, const void *ref,
+                                   const void *src, const float *base_plane,
+                                   const float *offsets, const float *depth_grid,
+                                   const float *Rs, const float *Ts, const void *cost_grad,
+                                   const int32_t *mask, void *ref_grad, void *src_grad,
+                                   float *depth_grad) {
+  const size_t need = chop_cost_volume_bwd16_workspace_bytes(B, H, W, C, N, srcH, srcW);
+  if (need > kScratchBytes) {
+    char buf[192];
+    snprintf(buf, sizeof buf,
+             "the gradient images need %zu bytes, the built-in scratch holds %zu: use "
+             "chop_cost_volume_bwd_16 with a workspace of the caller",
+             need, kScratchBytes);
+    return fail(CHOP_ERR_WORKSPACE, buf);
+  }
+  hipError_t err = hipSuccess;
+  void *ws = scratch_on_current_device(&err);
+  if (ws == nullptr) return launch_status(err, "address of the built-in scratch");
+  // (the launch clears the part of the scratch it accumulates into: launch_tiled_backward /
+  // launch_general_backward zero-fill both gradient images with a kernel before they add)
+  return chop_cost_volume_bwd_16(stream, storage, reduce, half_centor, B, H, W, C, D, N, srcH,
+                                 srcW, ref, src, base_plane, offsets, depth_grid, Rs, Ts,
+                                 cost_grad, mask, ref_grad, src_grad, depth_grad, ws,
+                                 kScratchBytes);
 }
 
 int chop_cost_volume_v2_fwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,

@@ -302,6 +302,24 @@ int chop_cost_volume_bwd_16(void *stream, int storage, int reduce, int half_cent
                             const void *cost_grad, const int32_t *mask, void *ref_grad,
                             void *src_grad, float *depth_grad, void *workspace,
                             size_t workspace_bytes);
+/* chop_cost_volume_bwd_16 for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in
+ * the reference.  Same arguments and results as chop_cost_volume_bwd_16 without the
+ * workspace: the fp32 gradient images live in a static device array of
+ * chop_static_scratch_bytes() (32 MiB) that every GPU the library runs on holds until the
+ * process ends; a shape whose chop_cost_volume_bwd16_workspace_bytes exceeds that is
+ * rejected with CHOP_ERR_WORKSPACE.  The call allocates and frees nothing.  All calls on one
+ * GPU share the array: calls that overlap in time on the same GPU (different streams or
+ * host threads) race and must be serialised by the caller. */
+size_t chop_static_scratch_bytes(void);
+int chop_cost_volume_bwd_16_static(void *stream, int storage, int reduce, int half_centor,
+                                   int64_t B, int64_t H, int64_t W, int64_t C, int64_t D,
+                                   int64_t N, int64_t srcH, int64_t srcW, const void *ref,
+                                   const void *src, const float *base_plane,
+                                   const float *offsets, const float *depth_grid,
+                                   const float *Rs, const float *Ts, const void *cost_grad,
+                                   const int32_t *mask, void *ref_grad, void *src_grad,
+                                   float *depth_grad);
 int chop_cost_volume_v2_fwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
                                int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
                                int64_t srcH, int64_t srcW, int groups, const void *ref,
