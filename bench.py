@@ -4,6 +4,13 @@ A step is one forward + one backward of the operator (through the C ABI) on one 
 synthetic input that is already resident in HBM.  Prints one JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2] [--no-cpu-baseline]
+                  [--no-configs]
+
+``value`` and ``ms_per_step`` are wall-clock over exactly K back-to-back steps.  The
+``roofline`` object is per call: HIP-event times of the dominant kernel's entry point with
+L2 and the memory-side cache overwritten before every call (cold), the back-to-back (warm)
+times beside them, and the rate a plain fill / copy reaches on this box in the same run.
+``configs`` holds the cold forward / backward times of all five benchmark configurations.
 
 The default run is the headline configuration (workload 2, MEAN).  ``--reduce MIN``,
 ``--aggregate`` (CostAggregate), ``--v3 GROUPS`` (CostVolumeV3) and ``--feature``
@@ -163,12 +170,17 @@ def cpu_baseline(wl, budget_s=12.0):
     cg = quantise(rng.standard_normal((wl.B, rows, wl.W, wl.D, wl.out_channels), dtype=np.float32),
                   wl.storage)
     times = []
+    out = None
+    if wl.op in ("v1", "v2"):  # the large outputs exist (and are touched) before the clock starts
+        oc = wl.out_channels
+        out = (np.zeros((wl.B, rows, wl.W, wl.D, oc), np.float32),
+               np.zeros((wl.B, rows, wl.W, wl.D, 1 if wl.reduce_method == "MEAN" else oc), np.int32))
     for _ in range(3):
         t0 = time.perf_counter()
         if wl.op == "v1":
             bp = t["base_plane"][:, sl]
             args = (ref, src, bp, t["offsets"], t["Rs"], t["Ts"])
-            _, mask = oracle.cost_volume_fwd(*args, wl.reduce_method, threads=threads)
+            _, mask = oracle.cost_volume_fwd(*args, wl.reduce_method, threads=threads, out=out)
             oracle.cost_volume_bwd(*args, cg, mask, wl.reduce_method, threads=threads)
         elif wl.op == "agg":
             bp = t["base_plane"][:, sl]
@@ -188,7 +200,8 @@ def cpu_baseline(wl, budget_s=12.0):
         else:
             dg = t["depth_grid"][:, sl]
             args = (ref, src, dg, t["Rs"], t["Ts"])
-            _, mask = oracle.cost_volume_v2_fwd(*args, wl.reduce_method, wl.groups, threads=threads)
+            _, mask = oracle.cost_volume_v2_fwd(*args, wl.reduce_method, wl.groups, threads=threads,
+                                                out=out)
             oracle.cost_volume_v2_bwd(*args, cg, mask, wl.reduce_method, wl.groups, threads=threads)
         times.append(time.perf_counter() - t0)
         if sum(times) > budget_s:
@@ -198,7 +211,86 @@ def cpu_baseline(wl, budget_s=12.0):
     vox = wl.B * rows * wl.W * wl.D
     return {"value": vox / med, "unit": "voxels/s", "cores": threads, "kind": "port",
             "sample": "%s rows 0..%d of %d (all views, all %d depths), fwd+bwd, median of %d, "
-                      "includes host allocation of outputs" % (wl.name, rows, wl.H, wl.D, len(times))}
+                      "cost and mask pre-allocated" % (wl.name, rows, wl.H, wl.D, len(times))}
+
+
+def timed_passes(torch, r, passes, scratch):
+    """`passes` forward + backward calls with HIP events on the launch stream around each
+    call.  With `scratch` (a 1 GiB buffer) every call is preceded by an overwrite of it, so
+    that L2 and the memory-side cache hold nothing of the workload: cold-cache times."""
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    marks = []
+    for _ in range(passes):
+        e0, e1, e2, e3 = ev(), ev(), ev(), ev()
+        if scratch is not None:
+            scratch.fill_(1.0)
+        e0.record()
+        r.forward()
+        e1.record()
+        if scratch is not None:
+            scratch.fill_(2.0)
+        e2.record()
+        r.backward()
+        e3.record()
+        marks.append((e0, e1, e2, e3))
+    torch.cuda.synchronize()
+    med = lambda v: sorted(v)[len(v) // 2]
+    return (med([m[0].elapsed_time(m[1]) for m in marks]),
+            med([m[2].elapsed_time(m[3]) for m in marks]))
+
+
+def stream_rates(torch):
+    """What this box's HBM gives a plain kernel, measured in this run: a 512 MiB fill
+    (write-only, the forward's pattern) and a 256 MiB copy (read + write)."""
+    n = 128 * 1024 * 1024
+    a = torch.empty(n, dtype=torch.float32, device="cuda:0")
+    b = torch.empty(n // 2, dtype=torch.float32, device="cuda:0")
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    fills, copies = [], []
+    for i in range(7):
+        e0, e1, e2 = ev(), ev(), ev()
+        e0.record()
+        a.fill_(float(i))
+        e1.record()
+        b.copy_(a[:n // 2])
+        e2.record()
+        torch.cuda.synchronize()
+        if i >= 2:
+            fills.append(e0.elapsed_time(e1))
+            copies.append(e1.elapsed_time(e2))
+    med = lambda v: sorted(v)[len(v) // 2]
+    del a, b
+    return {"fill_GBs": n * 4 / (med(fills) * 1e-3) / 1e9,
+            "copy_GBs": n * 4 / (med(copies) * 1e-3) / 1e9}  # copy: n/2 read + n/2 written
+
+
+def other_configs(torch, lib, make_workload, skip_index, scratch):
+    """Forward / backward event times of the BASELINE configurations the headline line is not
+    quoted on, each against its own algorithmic bytes (cold-cache, median of 5)."""
+    out = {}
+    for index in (1, 2, 3, 4, 5):
+        if index == skip_index:
+            continue
+        wl = make_workload(index, with_cost_grad=False)
+        r = Runner(wl, torch, lib)
+        for _ in range(2):
+            r.forward()
+            r.backward()
+        torch.cuda.synchronize()
+        fwd_ms, bwd_ms = timed_passes(torch, r, 5, scratch)
+        fwd_b, bwd_b = wl.algorithmic_bytes()
+        frac = lambda b, ms: b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+        out[wl.name] = {
+            "workload": "%s B%d N%d %dx%d C%d D%d %s" % (
+                {"v1": "CostVolume", "v2": "CostVolumeV2"}[wl.op], wl.B, wl.N, wl.H, wl.W, wl.C,
+                wl.D, wl.storage),
+            "voxels": wl.voxels, "forward_ms": fwd_ms, "backward_ms": bwd_ms,
+            "forward_frac": frac(fwd_b, fwd_ms), "backward_frac": frac(bwd_b, bwd_ms),
+            "fwd_bwd_frac": frac(fwd_b + bwd_b, fwd_ms + bwd_ms),
+            "voxels_per_s": wl.voxels / ((fwd_ms + bwd_ms) * 1e-3)}
+        del r
+        torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -208,6 +300,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the forward/backward times of the other BASELINE configurations")
     ap.add_argument("--reduce", choices=["MEAN", "MIN"], default="MEAN")
     ap.add_argument("--aggregate", action="store_true",
                     help="time CostAggregate on the workload's tensors (float32 CostVolume workloads)")
@@ -215,11 +309,6 @@ def main():
                     help="time CostVolumeV3 with this many channel groups on the workload's tensors")
     ap.add_argument("--feature", action="store_true",
                     help="time FeatureAggregate on the workload's tensors")
-    ap.add_argument("--flush-l2", action="store_true",
-                    help="overwrite a 1 GiB scratch buffer before every forward and every backward "
-                         "call, so that L2 and the memory-side cache hold nothing of the workload "
-                         "(the per-call event times then are cold-cache times; value and "
-                         "ms_per_step include the flushes and are not comparable)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
@@ -243,7 +332,6 @@ def main():
         wl.op = "v3" if a.v3 else "feat"
         wl.groups = a.v3 if a.v3 else 1
     r = Runner(wl, torch, lib)
-    ev = lambda: torch.cuda.Event(enable_timing=True)
     for _ in range(a.warmup):
         r.forward()
         r.backward()
@@ -256,38 +344,35 @@ def main():
             dst_buf.copy_(src_buf)
         torch.cuda.synchronize()
         del src_buf, dst_buf
-    marks = []
-    scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0") if a.flush_l2 else None
+    # the timed region: exactly `steps` steps, nothing else enqueued in between
     t0 = time.perf_counter()
     for _ in range(a.steps):
-        e0, e1, e2, e3 = ev(), ev(), ev(), ev()
-        if scratch is not None:
-            scratch.fill_(1.0)
-        e0.record()
         r.forward()
-        e1.record()
-        if scratch is not None:
-            scratch.fill_(2.0)
-        e2.record()
         r.backward()
-        e3.record()
-        marks.append((e0, e1, e2, e3))
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    fwd_ms = sum(m[0].elapsed_time(m[1]) for m in marks) / len(marks)
-    bwd_ms = sum(m[2].elapsed_time(m[3]) for m in marks) / len(marks)
     ms_per_step = wall * 1e3 / a.steps
+    # per-call times, outside the timed region: warm (back to back, as above) and cold (the
+    # caches overwritten before every call); the roofline line is the cold one
+    warm_fwd, warm_bwd = timed_passes(torch, r, max(a.steps, 5), None)
+    scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0")
+    fwd_ms, bwd_ms = timed_passes(torch, r, max(a.steps, 5), scratch)
     fwd_b, bwd_b = wl.algorithmic_bytes()
     dominant = "backward" if bwd_ms >= fwd_ms else "forward"
     d_ms, d_b = (bwd_ms, bwd_b) if dominant == "backward" else (fwd_ms, fwd_b)
+    w_ms = warm_bwd if dominant == "backward" else warm_fwd
     achieved = d_b / (d_ms * 1e-3) / 1e9
     traffic = None
-    try:  # measured with rocprofv3 counters in a separate run; the summary is under profiles/
+    traffic_source = None
+    try:  # HBM bytes per launch from rocprofv3 counters of a separate run of this command
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
             t = json.load(f)[wl.name if wl.op in ("v1", "v2") and a.reduce == "MEAN" else "-"][dominant]
         traffic = t["fetch_bytes"] + t["write_bytes"]
+        traffic_source = "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE/WRITE_SIZE of a separate run)"
     except (OSError, KeyError, ValueError):
         pass
+    rates = stream_rates(torch)
+    stream = rates["copy_GBs"] if dominant == "backward" else rates["fill_GBs"]
     out = {
         "metric": "cost-volume voxels/s (B*D*H*W) fwd+bwd",
         "value": wl.voxels / (ms_per_step * 1e-3),
@@ -300,15 +385,32 @@ def main():
                       "feat": "FeatureAggregate"}[wl.op],
             wl.B, wl.N, wl.H, wl.W,
             wl.C, wl.D, " G%d" % wl.groups if wl.op in ("v2", "v3") else "", wl.storage),
-            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True,
-                   **({"l2_flushed": True} if a.flush_l2 else {})},
+            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic,
+                     "timing": "HIP events on the launch stream, caches overwritten before each call, median",
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": {"forward": fwd_b, "backward": bwd_b},
                      "ms": {"forward": fwd_ms, "backward": bwd_ms},
-                     "fwd_bwd_frac": (fwd_b + bwd_b) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+                     "fwd_bwd_frac": (fwd_b + bwd_b) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "warm": {"ms": {"forward": warm_fwd, "backward": warm_bwd},
+                              "frac": d_b / (w_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                              "fwd_bwd_frac": (fwd_b + bwd_b) / ((warm_fwd + warm_bwd) * 1e-3) / 1e9
+                                              / HBM_PEAK_GBS},
+                     "measured_stream_GBs": stream,
+                     "measured_stream": {**rates, "used": "copy" if dominant == "backward" else "fill"},
+                     "frac_of_measured_stream": achieved / stream},
     }
+    if not a.no_configs and wl.op in ("v1", "v2") and a.reduce == "MEAN":
+        del r
+        torch.cuda.empty_cache()
+        out["configs"] = other_configs(torch, lib, make_workload, a.workload, scratch)
+        out["configs"][wl.name] = {
+            "workload": "headline", "voxels": wl.voxels, "forward_ms": fwd_ms, "backward_ms": bwd_ms,
+            "forward_frac": fwd_b / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "backward_frac": bwd_b / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "fwd_bwd_frac": out["roofline"]["fwd_bwd_frac"],
+            "voxels_per_s": wl.voxels / ((fwd_ms + bwd_ms) * 1e-3)}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))

@@ -92,27 +92,45 @@ def _check_v2(ref_image, src_images, depth_grid, Rs, Ts, groups):
     return B, H, W, C, N, depth_grid.shape[3]
 
 
+def _check_grid16(ref_image, src_images, depth_grid, Rs, Ts):
+    """Per-voxel hypotheses for the squared-difference op: an extension of the 16-bit storage
+    entry points (the registered CostVolume op only knows base_plane + offsets)."""
+    _require(ref_image.dtype in _STORAGE16,
+             "depth_grid with the squared-difference op needs float16 or bfloat16 features")
+    B, H, W, C, N = _check_common(ref_image, src_images, Rs, Ts)
+    _require(depth_grid.dim() == 4 and tuple(depth_grid.shape[:3]) == (B, H, W),
+             "depth_grid must have rank 4, and must compate to ref_image")
+    return B, H, W, C, N, depth_grid.shape[3]
+
+
 def cost_volume_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
-                    half_centor=True):
-    """Forward op without autograd: returns ``(cost [B,H,W,D,C], cost_mask int32)``."""
+                    half_centor=True, depth_grid=None):
+    """Forward op without autograd: returns ``(cost [B,H,W,D,C], cost_mask int32)``.
+    ``depth_grid`` ([B,H,W,D] float32, 16-bit feature storage only) replaces
+    ``base_plane + offsets`` (which may then be ``None``) by per-voxel hypotheses."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
     rdt = _real_dtype(dt)
     ref_image = _prep(ref_image, dt, dev, "ref_image")
     src_images = _prep(src_images, dt, dev, "src_images")
-    base_plane = _prep(base_plane, rdt, dev, "base_plane")
-    offsets = _prep(offsets, rdt, dev, "offsets")
     Rs, Ts = _prep(Rs, rdt, dev, "Rs"), _prep(Ts, rdt, dev, "Ts")
-    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, Rs, Ts)
+    if depth_grid is not None:
+        depth_grid = _prep(depth_grid, rdt, dev, "depth_grid")
+        B, H, W, C, N, D = _check_grid16(ref_image, src_images, depth_grid, Rs, Ts)
+        base_plane = offsets = None
+    else:
+        base_plane = _prep(base_plane, rdt, dev, "base_plane")
+        offsets = _prep(offsets, rdt, dev, "offsets")
+        B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, Rs, Ts)
     cost = torch.empty((B, H, W, D, C), dtype=dt, device=dev)
     mask = torch.empty((B, H, W, D, 1 if red == 0 else C), dtype=torch.int32, device=dev)
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
     if dt in _STORAGE16:
         rc = lib.chop_cost_volume_fwd_16(_stream(cost), _STORAGE16[dt], red, int(half_centor), *dims,
                                          _ptr(ref_image), _ptr(src_images), _ptr(base_plane),
-                                         _ptr(offsets), None, _ptr(Rs), _ptr(Ts), _ptr(cost),
-                                         _ptr(mask))
+                                         _ptr(offsets), _ptr(depth_grid), _ptr(Rs), _ptr(Ts),
+                                         _ptr(cost), _ptr(mask))
     else:
         fn = lib.chop_cost_volume_fwd_f32 if dt == torch.float32 else lib.chop_cost_volume_fwd_f64
         rc = fn(_stream(cost), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
@@ -122,36 +140,47 @@ def cost_volume_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_m
 
 
 def cost_volume_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_grad, cost_mask,
-                     reduce_method="MEAN", half_centor=True, need_depth_grad=True):
+                     reduce_method="MEAN", half_centor=True, need_depth_grad=True,
+                     depth_grid=None):
     """The ``CostVolumeGrad`` op: ``(ref_image_grad, src_images_grad, base_plane_grad)``.
     With ``need_depth_grad=False`` the third result is ``None`` and the kernels skip the
-    depth-derivative work (the registered op always computes it)."""
+    depth-derivative work (the registered op always computes it).  With ``depth_grid``
+    (16-bit feature storage only) the third result is the gradient of ``depth_grid``,
+    ``[B,H,W,D]``, zero on the voxels the mask skips."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
     rdt = _real_dtype(dt)
     ref_image = _prep(ref_image, dt, dev, "ref_image")
     src_images = _prep(src_images, dt, dev, "src_images")
-    base_plane = _prep(base_plane, rdt, dev, "base_plane")
-    offsets = _prep(offsets, rdt, dev, "offsets")
     rs, ts = _prep(rs, rdt, dev, "Rs"), _prep(ts, rdt, dev, "Ts")
     cost_grad = _prep(cost_grad, dt, dev, "cost_grad")
     cost_mask = _prep(cost_mask, torch.int32, dev, "cost_mask")
-    B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, rs, ts)
+    if depth_grid is not None:
+        depth_grid = _prep(depth_grid, rdt, dev, "depth_grid")
+        B, H, W, C, N, D = _check_grid16(ref_image, src_images, depth_grid, rs, ts)
+        base_plane = offsets = None
+    else:
+        base_plane = _prep(base_plane, rdt, dev, "base_plane")
+        offsets = _prep(offsets, rdt, dev, "offsets")
+        B, H, W, C, N, D = _check_v1(ref_image, src_images, base_plane, offsets, rs, ts)
     _require(tuple(cost_grad.shape) == (B, H, W, D, C),
              "cost_grad must have rank 5, and must compate to ref_image")
     _require(tuple(cost_mask.shape) == (B, H, W, D, 1 if red == 0 else C),
              "cost_mask must have rank 5, and must compate to ref_image")
     ref_grad = torch.empty_like(ref_image)
     src_grad = torch.empty_like(src_images)
-    bp_grad = torch.empty_like(base_plane) if need_depth_grad else None
+    bp_grad = None
+    if need_depth_grad:
+        bp_grad = torch.empty_like(depth_grid if depth_grid is not None else base_plane)
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
     if dt in _STORAGE16:
         need = lib.chop_cost_volume_bwd16_workspace_bytes(B, H, W, C, N, *dims[6:])
         ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
         rc = lib.chop_cost_volume_bwd_16(_stream(ref_grad), _STORAGE16[dt], red, int(half_centor),
                                          *dims, _ptr(ref_image), _ptr(src_images),
-                                         _ptr(base_plane), _ptr(offsets), None, _ptr(rs), _ptr(ts),
+                                         _ptr(base_plane), _ptr(offsets), _ptr(depth_grid),
+                                         _ptr(rs), _ptr(ts),
                                          _ptr(cost_grad), _ptr(cost_mask), _ptr(ref_grad),
                                          _ptr(src_grad), _ptr(bp_grad), _ptr(ws), need)
     else:

@@ -65,8 +65,19 @@ def _check(rc, name):
         raise ValueError("%s failed with oracle status %d" % (name, rc))
 
 
+def _outputs(out, cost_shape, mask_shape, dt):
+    """Fresh output arrays, or the caller's (already touched, so that a timed call does not
+    pay for the first-touch page faults of a new allocation)."""
+    if out is None:
+        return np.empty(cost_shape, dt), np.empty(mask_shape, np.int32)
+    cost, mask = out
+    assert cost.shape == cost_shape and cost.dtype == dt and cost.flags.c_contiguous
+    assert mask.shape == mask_shape and mask.dtype == np.int32 and mask.flags.c_contiguous
+    return cost, mask
+
+
 def cost_volume_fwd(ref, src, base_plane, offsets, Rs, Ts, reduce="MEAN", half_centor=True,
-                    threads=1):
+                    threads=1, out=None):
     dt = ref.dtype
     sfx = _sfx(dt)
     ref, src, base_plane, offsets, Rs, Ts = (_c(x, dt) for x in (ref, src, base_plane, offsets, Rs, Ts))
@@ -74,8 +85,7 @@ def cost_volume_fwd(ref, src, base_plane, offsets, Rs, Ts, reduce="MEAN", half_c
     N, sH, sW = src.shape[1:4]
     D = offsets.shape[1]
     r = _REDUCE[reduce]
-    cost = np.empty((B, H, W, D, C), dt)
-    mask = np.empty((B, H, W, D, 1 if r == 0 else C), np.int32)
+    cost, mask = _outputs(out, (B, H, W, D, C), (B, H, W, D, 1 if r == 0 else C), dt)
     fn = getattr(lib(), "chop_oracle_cost_volume_fwd_" + sfx)
     rc = fn(r, int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref), _p(src),
             _p(base_plane), _p(offsets), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
@@ -144,7 +154,7 @@ def cost_aggregate_bwd(ref, src, base_plane, offsets, Rs, Ts, cost_grad, mask, r
 
 
 def cost_volume_v2_fwd(ref, src, depth_grid, Rs, Ts, reduce="MEAN", groups=1, half_centor=True,
-                       threads=1):
+                       threads=1, out=None):
     dt = ref.dtype
     sfx = _sfx(dt)
     ref, src, depth_grid, Rs, Ts = (_c(x, dt) for x in (ref, src, depth_grid, Rs, Ts))
@@ -153,13 +163,50 @@ def cost_volume_v2_fwd(ref, src, depth_grid, Rs, Ts, reduce="MEAN", groups=1, ha
     D = depth_grid.shape[3]
     r = _REDUCE[reduce]
     G = int(groups)
-    cost = np.empty((B, H, W, D, max(G, 0)), dt)
-    mask = np.empty((B, H, W, D, 1 if r == 0 else max(G, 0)), np.int32)
+    cost, mask = _outputs(out, (B, H, W, D, max(G, 0)), (B, H, W, D, 1 if r == 0 else max(G, 0)), dt)
     fn = getattr(lib(), "chop_oracle_cost_volume_v2_fwd_" + sfx)
     rc = fn(r, int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW, G), _p(ref), _p(src),
             _p(depth_grid), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
     _check(rc, "cost_volume_v2_fwd")
     return cost, mask
+
+
+def cost_volume_grid_fwd(ref, src, depth_grid, Rs, Ts, reduce="MEAN", half_centor=True, threads=1):
+    """CostVolume's squared-difference reduce over per-voxel hypotheses ``depth_grid``."""
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, depth_grid, Rs, Ts = (_c(x, dt) for x in (ref, src, depth_grid, Rs, Ts))
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = depth_grid.shape[3]
+    r = _REDUCE[reduce]
+    cost, mask = _outputs(None, (B, H, W, D, C), (B, H, W, D, 1 if r == 0 else C), dt)
+    fn = getattr(lib(), "chop_oracle_cost_volume_grid_fwd_" + sfx)
+    rc = fn(r, int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref), _p(src),
+            _p(depth_grid), _p(Rs), _p(Ts), _p(cost), _p(mask), int(threads))
+    _check(rc, "cost_volume_grid_fwd")
+    return cost, mask
+
+
+def cost_volume_grid_bwd(ref, src, depth_grid, Rs, Ts, cost_grad, mask, reduce="MEAN",
+                         half_centor=True, threads=1):
+    dt = ref.dtype
+    sfx = _sfx(dt)
+    ref, src, depth_grid, Rs, Ts, cost_grad = (
+        _c(x, dt) for x in (ref, src, depth_grid, Rs, Ts, cost_grad))
+    mask = _c(mask, np.int32)
+    B, H, W, C = ref.shape
+    N, sH, sW = src.shape[1:4]
+    D = depth_grid.shape[3]
+    ref_grad = np.empty_like(ref)
+    src_grad = np.empty_like(src)
+    dg_grad = np.empty_like(depth_grid)
+    fn = getattr(lib(), "chop_oracle_cost_volume_grid_bwd_" + sfx)
+    rc = fn(_REDUCE[reduce], int(bool(half_centor)), *_i64(B, H, W, C, D, N, sH, sW), _p(ref),
+            _p(src), _p(depth_grid), _p(Rs), _p(Ts), _p(cost_grad), _p(mask), _p(ref_grad),
+            _p(src_grad), _p(dg_grad), int(threads))
+    _check(rc, "cost_volume_grid_bwd")
+    return ref_grad, src_grad, dg_grad
 
 
 def cost_volume_v2_bwd(ref, src, depth_grid, Rs, Ts, cost_grad, mask, reduce="MEAN", groups=1,

@@ -40,7 +40,8 @@ def test_oracle_exports():
     lib = oracle.lib()
     for sfx in ("f32", "f64"):
         for stem in ("cost_volume_fwd", "cost_volume_bwd", "cost_volume_v2_fwd", "cost_volume_v2_bwd",
-                     "cost_aggregate_fwd", "cost_aggregate_bwd", "sample_coords"):
+                     "cost_aggregate_fwd", "cost_aggregate_bwd", "sample_coords",
+                     "cost_volume_grid_fwd", "cost_volume_grid_bwd"):
             assert hasattr(lib, "chop_oracle_%s_%s" % (stem, sfx))
 
 

@@ -433,7 +433,114 @@ def test_golden_vectors(family):
             assert_backward_close(host(g), blob[name + "/out/" + k], tol)
 
 
+# ---- per-voxel hypotheses for the squared difference (cascade fine stage, exact form) ----------
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("storage", ["f16", "bf16"])
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+def test_v1_16bit_depth_grid(oracle, family, storage, reduce):
+    """chop_cost_volume_{fwd,bwd}_16 with a depth_grid: the cascade workload's multiplicative
+    hypotheses coarse * (1 + 0.02 k), N = 4 views, so that the per-voxel depth gradient of
+    the tiled kernels is added up over the view groups."""
+    _lib.load().chop_set_kernel_family(family)
+    wl = make_workload(3, hw=(40, 56))
+    t = wl.tensors
+    ref, src, cg = (quantise(t[k], storage) for k in ("ref", "src", "cost_grad"))
+    grid = t["depth_grid"]
+    assert grid.shape == (1, 40, 56, 32)
+    want_cost, want_mask = oracle.cost_volume_grid_fwd(ref, src, grid, t["Rs"], t["Ts"], reduce,
+                                                       threads=8)
+    td = TORCH_DTYPE[storage]
+    d_ref, d_src, d_grid, d_rs, d_ts = dev(ref, td), dev(src, td), dev(grid), dev(t["Rs"]), dev(t["Ts"])
+    cost, mask = chop.cost_volume_raw(d_ref, d_src, None, None, d_rs, d_ts, reduce, depth_grid=d_grid)
+    _assert_family(family)
+    assert np.array_equal(host(mask), want_mask)
+    if reduce == "MEAN":
+        _assert_16bit_close(host(cost), want_cost, storage)
+    else:  # rows no view reaches keep the float maximum, which does not fit 16 bits
+        ok = want_mask >= 0
+        np.testing.assert_allclose(host(cost)[ok], want_cost[ok], rtol=1e-2,
+                                   atol=1e-2 * rms(want_cost[ok]))
+    want = oracle.cost_volume_grid_bwd(ref, src, grid, t["Rs"], t["Ts"], cg, want_mask, reduce)
+    got = chop.cost_volume_grad(d_ref, d_src, None, None, d_rs, d_ts, dev(cg, td), dev(want_mask),
+                                reduce, depth_grid=d_grid)
+    _assert_family(family)
+    assert got[2].shape == grid.shape and got[2].dtype == torch.float32
+    for g, w in zip(got, want):
+        _assert_16bit_close(host(g), w, storage)
+    # no depth gradient wanted: the other two are unchanged
+    two = chop.cost_volume_grad(d_ref, d_src, None, None, d_rs, d_ts, dev(cg, td), dev(want_mask),
+                                reduce, need_depth_grad=False, depth_grid=d_grid)
+    assert two[2] is None
+    _assert_16bit_close(host(two[0]), want[0], storage)
+    _assert_16bit_close(host(two[1]), want[1], storage)
+
+
+def test_depth_grid_needs_16bit_storage():
+    wl = make_workload(3, hw=(8, 8))
+    t = wl.tensors
+    with pytest.raises(chop.InvalidArgumentError):
+        chop.cost_volume_raw(dev(t["ref"]), dev(t["src"]), None, None, dev(t["Rs"]), dev(t["Ts"]),
+                             depth_grid=dev(t["depth_grid"]))
+
+
 # ---- full benchmark sizes -----------------------------------------------------------------------
+@pytest.mark.parametrize("form", ["plane", "grid"])
+def test_cascade_fine_full_size(oracle, form):
+    """Benchmark configuration 3 at its real size (f16 storage, B1 N4 256x320 C16 D32), both
+    forms: base_plane + additive offsets (the registered op's) and the exact per-pixel
+    multiplicative hypotheses through depth_grid."""
+    wl = make_workload(3)
+    t = wl.tensors
+    ref, src, cg = (quantise(t[k], "f16") for k in ("ref", "src", "cost_grad"))
+    td = torch.float16
+    d_ref, d_src, d_rs, d_ts = dev(ref, td), dev(src, td), dev(t["Rs"]), dev(t["Ts"])
+    if form == "plane":
+        args = (ref, src, t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+        want_cost, want_mask = oracle.cost_volume_fwd(*args, threads=16)
+        want = oracle.cost_volume_bwd(*args, cg, want_mask, threads=16)
+        cost, mask = chop.cost_volume_raw(d_ref, d_src, dev(t["base_plane"]), dev(t["offsets"]), d_rs, d_ts)
+        _assert_family(0)
+        got = chop.cost_volume_grad(d_ref, d_src, dev(t["base_plane"]), dev(t["offsets"]), d_rs, d_ts,
+                                    dev(cg, td), mask)
+    else:
+        args = (ref, src, t["depth_grid"], t["Rs"], t["Ts"])
+        want_cost, want_mask = oracle.cost_volume_grid_fwd(*args, threads=16)
+        want = oracle.cost_volume_grid_bwd(*args, cg, want_mask, threads=16)
+        d_grid = dev(t["depth_grid"])
+        cost, mask = chop.cost_volume_raw(d_ref, d_src, None, None, d_rs, d_ts, depth_grid=d_grid)
+        _assert_family(0)
+        got = chop.cost_volume_grad(d_ref, d_src, None, None, d_rs, d_ts, dev(cg, td), mask,
+                                    depth_grid=d_grid)
+    _assert_family(0)
+    assert cost.shape == (1, 256, 320, 32, 16)
+    assert np.array_equal(host(mask), want_mask)
+    _assert_16bit_close(host(cost), want_cost, "f16")
+    for g, w in zip(got, want):
+        _assert_16bit_close(host(g), w, "f16")
+
+
+def test_group_correlation_full_size(oracle):
+    """Benchmark configuration 4 at its real size (bf16 storage, B2 N4 512x640 C8 G4 D8)."""
+    wl = make_workload(4)
+    t = wl.tensors
+    ref, src, cg = (quantise(t[k], "bf16") for k in ("ref", "src", "cost_grad"))
+    args = (ref, src, t["depth_grid"], t["Rs"], t["Ts"])
+    want_cost, want_mask = oracle.cost_volume_v2_fwd(*args, "MEAN", 4, threads=16)
+    want = oracle.cost_volume_v2_bwd(*args, cg, want_mask, "MEAN", 4, threads=16)
+    td = torch.bfloat16
+    ins = [dev(ref, td), dev(src, td), dev(t["depth_grid"]), dev(t["Rs"]), dev(t["Ts"])]
+    cost, mask = chop.cost_volume_v2_raw(*ins, "MEAN", 4)
+    _assert_family(0)
+    assert cost.shape == (2, 512, 640, 8, 4)
+    assert np.array_equal(host(mask), want_mask)
+    _assert_16bit_close(host(cost), want_cost, "bf16")
+    got = chop.cost_volume_grad_v2(*ins, dev(cg, td), mask, "MEAN", 4)
+    _assert_family(0)
+    for g, w in zip(got, want):
+        _assert_16bit_close(host(g), w, "bf16")
+
+
+
 def test_mvsnet_stage_full_size(oracle):
     """Benchmark configuration 2 at its real size, forward and backward, against the oracle
     (the oracle takes a few seconds on the box's host cores)."""

@@ -164,3 +164,44 @@ def test_v2_mean_linear_in_ref(oracle):
     r2, s2, _ = oracle.cost_volume_v2_bwd(3 * t["ref"], t["src"], dg, t["Rs"], t["Ts"], cg, m1, "MEAN", 2)
     np.testing.assert_allclose(r1, r2, rtol=1e-12, atol=1e-14)
     np.testing.assert_allclose(3 * s1, s2, rtol=1e-12, atol=1e-14)
+
+
+# ---- squared difference over a depth grid ------------------------------------------------------
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+def test_grid_entry_equals_the_plane_entry_bit_for_bit(oracle, dtype, reduce):
+    """chop_oracle_cost_volume_grid_* is the pinned CostVolume oracle with another depth
+    source.  On depth_grid = base_plane + offsets (formed in the same precision, the kernel's
+    own expression, cost_volume_kernels_gpu.cu.cc:64) every voxel sees the same depth, so cost,
+    mask, ref_grad and src_grad must equal the pinned functions' to the bit, and the per-voxel
+    depth gradient must add up, in depth order, to the per-pixel one."""
+    t = reference_test_case(3, B=2, N=3, H=12, W=18, C=5, D=10, dtype=dtype, seed=21)
+    args = (t["ref"], t["src"], t["base_plane"], t["offsets"], t["Rs"], t["Ts"])
+    grid = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(dtype)
+    want_cost, want_mask = oracle.cost_volume_fwd(*args, reduce)
+    cost, mask = oracle.cost_volume_grid_fwd(t["ref"], t["src"], grid, t["Rs"], t["Ts"], reduce)
+    assert np.array_equal(mask, want_mask)
+    assert np.array_equal(cost.view(np.uint8), want_cost.view(np.uint8))
+    assert (want_mask > 0).any() if reduce == "MEAN" else (want_mask >= 0).any()
+    rng = np.random.default_rng(5)
+    cg = rng.standard_normal(cost.shape).astype(dtype)
+    want = oracle.cost_volume_bwd(*args, cg, want_mask, reduce)
+    got = oracle.cost_volume_grid_bwd(t["ref"], t["src"], grid, t["Rs"], t["Ts"], cg, want_mask, reduce)
+    assert np.array_equal(got[0], want[0])
+    assert np.array_equal(got[1], want[1])
+    total = np.zeros(want[2].shape[:3], dtype)
+    for d in range(grid.shape[3]):  # the plane entry adds its voxels up in this order (:454)
+        total = (total + got[2][..., d]).astype(dtype)
+    assert np.array_equal(total, want[2][..., 0])
+    # voxels the mask skips get a zero, as in CostVolumeGradV2 (cost_volume_kernels_gpu_v2.cu.cc:375-378)
+    skipped = (want_mask[..., 0] <= 0) if reduce == "MEAN" else (want_mask[..., 0] < 0)
+    assert skipped.any() and not got[2][skipped].any()
+    # several threads: the same forward, the same pixel-owned gradients
+    cost4, mask4 = oracle.cost_volume_grid_fwd(t["ref"], t["src"], grid, t["Rs"], t["Ts"], reduce,
+                                               threads=4)
+    assert np.array_equal(cost4, cost) and np.array_equal(mask4, mask)
+    got4 = oracle.cost_volume_grid_bwd(t["ref"], t["src"], grid, t["Rs"], t["Ts"], cg, want_mask,
+                                       reduce, threads=4)
+    assert np.array_equal(got4[0], got[0]) and np.array_equal(got4[2], got[2])
+    np.testing.assert_allclose(got4[1], got[1], rtol=1e-5 if dtype == np.float32 else 1e-12,
+                               atol=1e-5 if dtype == np.float32 else 1e-12)
