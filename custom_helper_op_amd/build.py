@@ -15,7 +15,7 @@ LIB = os.path.join(HERE, "libchop_costvol.so")
 SOURCES = ["tiled_f32_fwd_wide.hip", "tiled_f32_bwd_wide.hip", "tiled_f32_fwd_narrow.hip",
            "tiled_f32_bwd_narrow.hip", "tiled_f16_fwd.hip", "tiled_f16_bwd.hip",
            "tiled_bf16_fwd.hip", "tiled_bf16_bwd.hip", "api.hip", "general.hip", "v3_feature.hip",
-           "epilogue.hip", "tiled.hip"]
+           "epilogue.hip", "tiled.hip", "strip.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off", "-fno-fast-math",

@@ -101,6 +101,10 @@ int forward(void *stream, int reduce, int half_centor, const Dims &d, int groups
     g_last_family = 2;
     return launch_status(launch_tiled_forward(a, s), "tiled forward launch");
   }
+  if (g_kernel_family != 1 && strip_supported(a)) {
+    g_last_family = 3;
+    return launch_status(launch_strip_forward(a, s), "strip forward launch");
+  }
   g_last_family = 1;
   return launch_status(launch_general_forward(a, s), "general forward launch");
 }
@@ -166,6 +170,10 @@ int backward(void *stream, int reduce, int half_centor, const Dims &d, int group
   if (g_kernel_family == 0 && work && tiled_backward_supported(a)) {
     g_last_family = 2;
     return launch_status(launch_tiled_backward(a, s), "tiled backward launch");
+  }
+  if (g_kernel_family != 1 && work && strip_supported(a)) {
+    g_last_family = 3;
+    return launch_status(launch_strip_backward(a, s), "strip backward launch");
   }
   g_last_family = 1;
   return launch_status(launch_general_backward(a, s), "general backward launch");
@@ -324,7 +332,7 @@ const char *chop_last_error_string(void) { return g_last_error.c_str(); }
 
 int chop_set_kernel_family(int family) {
   const int prev = g_kernel_family;
-  g_kernel_family = family == 1 ? 1 : 0;
+  g_kernel_family = family == 1 || family == 2 ? family : 0;
   return prev;
 }
 

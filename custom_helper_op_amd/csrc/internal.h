@@ -94,6 +94,16 @@ hipError_t launch_general_forward(const Args<S> &a, hipStream_t stream);
 template <typename S>
 hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream);
 
+// Strip kernels: one wavefront per strip of pixels, one lane per channel, depth innermost.
+// CostVolume and CostVolumeV2 with up to 64 channels, any view count, all storage types:
+// what the tiled kernels decline (float64, channel counts other than 4 x 2^k) runs here.
+template <typename S>
+bool strip_supported(const Args<S> &a);
+template <typename S>
+hipError_t launch_strip_forward(const Args<S> &a, hipStream_t stream);
+template <typename S>
+hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream);
+
 // CostVolumeV3 (corr = BEST_GROUP_PAIR) and FeatureAggregate (corr = WARP_ONLY; `ref` unused,
 // `cost` = mapped_feature [B,H,W,D,N,C], `mask` = mapped_mask [B,H,W,D,N]): float and double.
 template <typename S>

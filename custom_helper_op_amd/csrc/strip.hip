@@ -1,0 +1,467 @@
+// Strip kernels: the wave-per-pixel-strip decomposition for every shape the tiled kernels do
+// not take -- float64 (the element type of the reference's own tests), channel counts that
+// are not 4 x a power of two (the reference tests use 3, 5 and 9), any number of views -- for
+// CostVolume and CostVolumeV2, both reduces, all four storage types, up to 64 channels.
+//
+// A workgroup is one wavefront.  It owns 64/LPP consecutive pixels (LPP = the power of two
+// >= C: one lane per channel, so a tap read or a cost-row write of a pixel is one contiguous
+// C-element segment) and one segment of the depth hypotheses, walked in chunks of kDB depths
+// with the views as the middle loop:
+//   phase 1  the first kDB lanes of a pixel reproject the chunk's depths into the view (the
+//            bit-exact code of warp.h) and leave one record per (pixel, depth) in LDS;
+//   phase 2  every lane walks the chunk's depths for its channel; the four taps stay in
+//            registers while consecutive depths fall into the same texel cell.
+// Forward: the arithmetic is the reference's literal operand order, every operation rounded
+// separately (cost_volume_kernels_gpu.cu.cc:33-228, cost_volume_kernels_gpu_v2.cu.cc:33-235),
+// views and channels summed in the reference's order, so float and double results are
+// bit-identical to a plain IEEE CPU evaluation, as with the general kernels.
+// Backward (:342-577, v2 :349-601): ref_grad and the base-plane gradient are pixel-owned and
+// stay in registers; the source-gradient contributions of a run of depths that share a cell
+// are merged in registers and leave as one atomic add per tap and channel when the cell
+// changes (the reference issues one per voxel); the per-voxel depth gradient is summed over
+// the pixel's lanes in registers and stored once.
+#include <type_traits>
+
+#include "internal.h"
+
+namespace chop {
+
+namespace {
+
+constexpr int kDB = 8;  // depths per chunk
+
+struct StripGeom {
+  int lpp_shift;        // log2(LPP)
+  int nseg, seg;        // depth segments, depths per segment (a multiple of kDB)
+  int64_t tiles;        // ceil(B*H*W / PPW)
+};
+
+__device__ __forceinline__ void strip_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Sum over the 2^shift consecutive lanes of a pixel, left in every one of them.
+template <typename R>
+__device__ __forceinline__ R pixel_sum(R v, int shift) {
+  for (int s = 0; s < shift; ++s) v += __shfl_xor(v, 1 << s, 64);
+  return v;
+}
+
+template <typename R>
+struct StripPixel {
+  int64_t pix;
+  int b;
+  R ref_w, ref_h;
+  bool ok;
+};
+
+template <typename S>
+__device__ __forceinline__ StripPixel<typename Storage<S>::Real> strip_pixel(const Args<S> &a,
+                                                                              int64_t pix) {
+  using R = typename Storage<S>::Real;
+  StripPixel<R> px;
+  const int64_t npix = a.pixels();
+  px.ok = pix < npix;
+  px.pix = px.ok ? pix : npix - 1;  // clamp: loads stay in range, stores are predicated
+  const int64_t row = px.pix / a.W;
+  const int w = (int)(px.pix - row * a.W);
+  px.b = (int)(row / a.H);
+  const int h = (int)(row - (int64_t)px.b * a.H);
+  px.ref_w = static_cast<R>(w) + a.half;
+  px.ref_h = static_cast<R>(h) + a.half;
+  return px;
+}
+
+// LDS of one wavefront: kDB records per pixel; a record is addressed [field][pixel*kDB + j].
+template <typename R>
+struct StripRecords {
+  R *f;      // NF fields of 64/LPP*kDB values each
+  int *off;  // tap offset inside the view, -1: nothing to do
+  int stride;
+  __device__ __forceinline__ R &at(int field, int idx) { return f[field * stride + idx]; }
+};
+
+template <typename R, int NF>
+__device__ __forceinline__ StripRecords<R> strip_records(unsigned char *smem, int ppw) {
+  StripRecords<R> r;
+  r.stride = ppw * kDB;
+  r.f = reinterpret_cast<R *>(smem);
+  r.off = reinterpret_cast<int *>(smem + (size_t)NF * r.stride * sizeof(R));
+  return r;
+}
+
+template <typename R>
+constexpr size_t strip_lds_bytes(int nf, int ppw) {
+  return (size_t)ppw * kDB * (nf * sizeof(R) + sizeof(int)) + 64 * sizeof(R);
+}
+
+// ------------------------------------------------------------------------------------------
+// Forward
+// ------------------------------------------------------------------------------------------
+template <typename S, int CORR, int REDUCE>
+__global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, const StripGeom g) {
+  using R = typename Storage<S>::Real;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x, lpp = 1 << g.lpp_shift, ppw = 64 >> g.lpp_shift;
+  const int p = lane >> g.lpp_shift, cl = lane & (lpp - 1);
+  const int64_t tile = (int64_t)blockIdx.x / g.nseg;
+  const int segi = (int)((int64_t)blockIdx.x - tile * g.nseg);
+  const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int OC = CORR ? a.groups : C;
+  const int sub = CORR ? C / a.groups : 1;
+  const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
+  const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
+  const bool ch_ok = cl < C, out_ok = px.ok && cl < OC;
+  const R ref_c = ch_ok ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
+  const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
+  const int64_t row_step = (int64_t)srcW * C;
+  StripRecords<R> rec = strip_records<R, 4>(smem, ppw);
+  R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw)) - 64;  // CORR: products of a pixel
+  const int ridx = p * kDB;
+
+  for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
+    R acc[kDB];
+    int arg[kDB], kcnt[kDB];
+#pragma unroll
+    for (int jj = 0; jj < kDB; ++jj) {
+      acc[jj] = REDUCE == 0 ? R(0) : (CORR ? Limits<R>::min_positive() : Limits<R>::max());
+      arg[jj] = -1;
+      kcnt[jj] = 0;
+    }
+    for (int n = 0; n < N; ++n) {
+      const int64_t cam = (int64_t)px.b * N + n;
+      strip_sync();  // the records of the view before have been read
+      for (int j = cl; j < kDB; j += lpp) {
+        const int d = d0 + j;
+        int off = -1;
+        Sample<R> s;
+        s.k00 = s.k01 = s.k11 = s.k10 = R(0);
+        if (d < d_hi) {
+          const R depth = a.depth_grid ? a.depth_grid[px.pix * D + d]
+                                       : base + a.offsets[(int64_t)px.b * D + d];
+          project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
+          if (s.state == 2) off = (s.fh * srcW + s.fw) * C;
+        }
+        rec.off[ridx + j] = off;
+        rec.at(0, ridx + j) = s.k00;
+        rec.at(1, ridx + j) = s.k01;
+        rec.at(2, ridx + j) = s.k11;
+        rec.at(3, ridx + j) = s.k10;
+      }
+      strip_sync();
+      const S *view = a.src + cam * srcH * srcW * C + (ch_ok ? cl : 0);
+      int cur = -1;
+      R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
+#pragma unroll
+      for (int jj = 0; jj < kDB; ++jj) {
+        const int off = rec.off[ridx + jj];
+        if (off < 0) continue;
+        if (off != cur) {
+          cur = off;
+          const S *q = view + off;
+          v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
+          v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
+        }
+        const R smp = rec.at(0, ridx + jj) * v00 + rec.at(1, ridx + jj) * v01 +
+                      rec.at(2, ridx + jj) * v11 + rec.at(3, ridx + jj) * v10;
+        R val;
+        if (CORR == 0) {
+          const R diff = smp - ref_c;
+          val = diff * diff;
+        } else {
+          // the group's products, added up from zero in channel order by the group's lane
+          s_prod[lane] = smp * ref_c;
+          strip_sync();
+          val = R(0);
+          if (cl < OC)
+            for (int c = 0; c < sub; ++c) val += s_prod[p * lpp + cl * sub + c];
+          strip_sync();
+        }
+        if (REDUCE == 0) {
+          acc[jj] += val;
+        } else if (CORR ? (acc[jj] < val) : (acc[jj] > val)) {
+          acc[jj] = val;
+          arg[jj] = n;
+        }
+        ++kcnt[jj];
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < kDB; ++jj) {
+      const int d = d0 + jj;
+      if (d >= d_hi) break;
+      const int64_t i = px.pix * D + d;
+      if (REDUCE == 0) {
+        if (kcnt[jj] > 0) acc[jj] = acc[jj] / static_cast<R>(kcnt[jj]);
+        if (px.ok && cl == 0) a.mask[i] = kcnt[jj];
+      } else if (out_ok) {
+        a.mask[i * OC + cl] = arg[jj];
+      }
+      if (out_ok) Storage<S>::store(a.cost + i * OC + cl, acc[jj]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Backward
+// ------------------------------------------------------------------------------------------
+template <typename S, int CORR, int REDUCE>
+__global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, const StripGeom g) {
+  using R = typename Storage<S>::Real;
+  using Acc = typename std::conditional<sizeof(S) == 2, float, S>::type;
+  extern __shared__ __align__(16) unsigned char smem[];
+  Acc *ref_grad = sizeof(S) == 2 ? (Acc *)a.ref_grad_acc : (Acc *)a.ref_grad;
+  Acc *src_grad = sizeof(S) == 2 ? (Acc *)a.src_grad_acc : (Acc *)a.src_grad;
+  const int lane = threadIdx.x, lpp = 1 << g.lpp_shift, ppw = 64 >> g.lpp_shift;
+  const int p = lane >> g.lpp_shift, cl = lane & (lpp - 1);
+  const int64_t tile = (int64_t)blockIdx.x / g.nseg;
+  const int segi = (int)((int64_t)blockIdx.x - tile * g.nseg);
+  const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
+  const int OC = CORR ? a.groups : C;
+  const int sub = CORR ? C / a.groups : 1;
+  const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
+  const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
+  const bool ch_ok = cl < C && px.ok;
+  const int oc = CORR ? (ch_ok ? cl / sub : 0) : (ch_ok ? cl : 0);
+  const R ref_c = ch_ok ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
+  const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
+  const bool per_voxel = a.depth_grid != nullptr, want_depth = a.depth_grad != nullptr;
+  const int64_t row_step = (int64_t)srcW * C;
+  // fields: the four weights, dh, dw, the two depth-chain factors, the view count as a real
+  StripRecords<R> rec = strip_records<R, 9>(smem, ppw);
+  const int ridx = p * kDB;
+  R racc = R(0), dpart = R(0);
+
+  for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
+    R dvox[kDB];
+#pragma unroll
+    for (int jj = 0; jj < kDB; ++jj) dvox[jj] = R(0);
+    for (int n = 0; n < N; ++n) {
+      const int64_t cam = (int64_t)px.b * N + n;
+      strip_sync();
+      for (int j = cl; j < kDB; j += lpp) {
+        const int d = d0 + j;
+        int off = -1;
+        Sample<R> s;
+        s.k00 = s.k01 = s.k11 = s.k10 = s.dh = s.dw = R(0);
+        R fh = R(0), fw = R(0), cnt = R(1);
+        if (d < d_hi && px.ok) {
+          const int64_t i = px.pix * D + d;
+          const int32_t m0 = a.mask_in[REDUCE == 0 ? i : i * OC];
+          // MEAN skips a voxel no view reached (:367), MIN one whose first entry is negative (:484)
+          if (REDUCE == 0 ? (m0 > 0) : (m0 >= 0)) {
+            const R depth = per_voxel ? a.depth_grid[i] : base + a.offsets[(int64_t)px.b * D + d];
+            project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
+            if (s.state == 2) {
+              off = (s.fh * srcW + s.fw) * C;
+              const R zz = s.z * s.z;
+              fh = (s.h_coef * s.z - s.z_coef * s.h3d) / zz;
+              fw = (s.w_coef * s.z - s.z_coef * s.w3d) / zz;
+              cnt = static_cast<R>(m0);
+            }
+          }
+        }
+        rec.off[ridx + j] = off;
+        rec.at(0, ridx + j) = s.k00;
+        rec.at(1, ridx + j) = s.k01;
+        rec.at(2, ridx + j) = s.k11;
+        rec.at(3, ridx + j) = s.k10;
+        rec.at(4, ridx + j) = s.dh;
+        rec.at(5, ridx + j) = s.dw;
+        rec.at(6, ridx + j) = fh;
+        rec.at(7, ridx + j) = fw;
+        rec.at(8, ridx + j) = cnt;
+      }
+      strip_sync();
+      const int64_t view_off = cam * srcH * srcW * C + (ch_ok ? cl : 0);
+      const S *view = a.src + view_off;
+      Acc *gview = src_grad + view_off;
+      int cur = -1;
+      R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
+      R g00 = R(0), g01 = R(0), g11 = R(0), g10 = R(0);
+      auto flush = [&]() {
+        if (cur >= 0 && ch_ok) {
+          Acc *q = gview + cur;
+          if (g00 != R(0)) atomic_add(q, (Acc)g00);
+          if (g01 != R(0)) atomic_add(q + C, (Acc)g01);
+          if (g11 != R(0)) atomic_add(q + C + row_step, (Acc)g11);
+          if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
+        }
+        g00 = g01 = g11 = g10 = R(0);
+      };
+#pragma unroll
+      for (int jj = 0; jj < kDB; ++jj) {
+        const int off = rec.off[ridx + jj];
+        if (off < 0) continue;
+        const int64_t i = px.pix * D + d0 + jj;
+        if (off != cur) {
+          flush();
+          cur = off;
+          const S *q = view + off;
+          v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
+          v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
+        }
+        if (!ch_ok) continue;
+        if (REDUCE != 0 && a.mask_in[i * OC + oc] != n) continue;  // another view won (:553)
+        const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
+                k10 = rec.at(3, ridx + jj);
+        const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
+        const R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
+        const R cnt = rec.at(8, ridx + jj);
+        R gv;
+        if (CORR == 0) {
+          const R diff = smp - ref_c;
+          gv = REDUCE == 0 ? R(2) * diff * cg / cnt : R(2) * diff * cg;  // :439, :560
+          racc += -gv;
+        } else {
+          gv = REDUCE == 0 ? cg / cnt : cg;  // v2 :461, :583
+          racc += gv * smp;
+          gv = gv * ref_c;
+        }
+        g00 += gv * k00;
+        g01 += gv * k01;
+        g11 += gv * k11;
+        g10 += gv * k10;
+        if (want_depth) {
+          const R t1 = v11 - v10 - v01 + v00;
+          const R h_grad = gv * (t1 * rec.at(5, ridx + jj) + v10 - v00);
+          const R w_grad = gv * (t1 * rec.at(4, ridx + jj) + v01 - v00);
+          const R dl = rec.at(6, ridx + jj) * h_grad + rec.at(7, ridx + jj) * w_grad;
+          if (per_voxel)
+            dvox[jj] += dl;
+          else
+            dpart += dl;
+        }
+      }
+      flush();
+    }
+    if (per_voxel && want_depth) {
+#pragma unroll
+      for (int jj = 0; jj < kDB; ++jj) {
+        const R tot = pixel_sum(dvox[jj], g.lpp_shift);
+        const int d = d0 + jj;
+        // every voxel is stored, zeros on the ones the mask skips (v2 :375-378, :477)
+        if (d < d_hi && px.ok && cl == 0) a.depth_grad[px.pix * D + d] = tot;
+      }
+    }
+  }
+  if (ch_ok) {
+    Acc *q = ref_grad + px.pix * C + cl;
+    if (g.nseg == 1)
+      *q = (Acc)racc;
+    else
+      atomic_add(q, (Acc)racc);
+  }
+  if (!per_voxel && want_depth) {
+    const R tot = pixel_sum(dpart, g.lpp_shift);
+    if (px.ok && cl == 0) {
+      if (g.nseg == 1)
+        a.depth_grad[px.pix] = tot;
+      else
+        atomic_add(a.depth_grad + px.pix, tot);
+    }
+  }
+}
+
+template <typename S>
+StripGeom strip_geometry(const Args<S> &a) {
+  StripGeom g;
+  g.lpp_shift = 0;
+  while ((1 << g.lpp_shift) < a.C) ++g.lpp_shift;
+  const int ppw = 64 >> g.lpp_shift;
+  g.tiles = (a.pixels() + ppw - 1) / ppw;
+  // enough wavefronts to fill 256 compute units several times over, segments of whole chunks
+  int nseg = 1;
+  while (nseg < 16 && g.tiles * nseg < 256 * 16 && a.D / (nseg * 2) >= kDB) nseg *= 2;
+  const int per = (int)((a.D + nseg - 1) / nseg);
+  g.seg = (per + kDB - 1) / kDB * kDB;
+  g.nseg = (int)((a.D + g.seg - 1) / g.seg);
+  return g;
+}
+
+}  // namespace
+
+template <typename S>
+bool strip_supported(const Args<S> &a) {
+  if (a.corr != SQUARED_DIFFERENCE && a.corr != GROUP_CORRELATION) return false;
+  if (a.C < 1 || a.C > 64 || a.N < 1 || a.D < 1 || a.pixels() < 1) return false;
+  if (a.corr == GROUP_CORRELATION && (a.groups < 1 || a.C % a.groups != 0)) return false;
+  if (a.srcH < 2 || a.srcW < 2) return false;                   // no sample can be accepted
+  if (a.srcH * a.srcW * a.C >= (int64_t)1 << 31) return false;  // 32-bit offsets inside a view
+  const StripGeom g = strip_geometry(a);
+  return g.tiles * g.nseg < (int64_t)1 << 31;
+}
+
+template <typename S>
+hipError_t launch_strip_forward(const Args<S> &a, hipStream_t stream) {
+  using R = typename Storage<S>::Real;
+  const StripGeom g = strip_geometry(a);
+  const size_t smem = strip_lds_bytes<R>(4, 64 >> g.lpp_shift);
+  const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
+  if (a.corr == SQUARED_DIFFERENCE) {
+    if (a.reduce == 0)
+      strip_forward_kernel<S, 0, 0><<<grid, block, smem, stream>>>(a, g);
+    else
+      strip_forward_kernel<S, 0, 1><<<grid, block, smem, stream>>>(a, g);
+  } else {
+    if (a.reduce == 0)
+      strip_forward_kernel<S, 1, 0><<<grid, block, smem, stream>>>(a, g);
+    else
+      strip_forward_kernel<S, 1, 1><<<grid, block, smem, stream>>>(a, g);
+  }
+  return hipGetLastError();
+}
+
+template <typename S>
+hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
+  using R = typename Storage<S>::Real;
+  const StripGeom g = strip_geometry(a);
+  const int64_t n_ref = a.pixels() * a.C;
+  const int64_t n_src = a.B * a.N * a.srcH * a.srcW * a.C;
+  hipError_t err;
+  // the scatter target starts from zero; the pixel-owned outputs only when several depth
+  // segments add into them (otherwise the kernel stores every element once)
+  void *src_img = sizeof(S) == 2 ? (void *)a.src_grad_acc : (void *)a.src_grad;
+  void *ref_img = sizeof(S) == 2 ? (void *)a.ref_grad_acc : (void *)a.ref_grad;
+  const size_t acc_size = sizeof(S) == 2 ? 4 : sizeof(S);
+  if ((err = launch_fill_zero(src_img, (size_t)n_src * acc_size, stream)) != hipSuccess) return err;
+  if (g.nseg > 1) {
+    if ((err = launch_fill_zero(ref_img, (size_t)n_ref * acc_size, stream)) != hipSuccess) return err;
+    if (a.depth_grid == nullptr && a.depth_grad != nullptr &&
+        (err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(R), stream)) != hipSuccess)
+      return err;
+  }
+  const size_t smem = strip_lds_bytes<R>(9, 64 >> g.lpp_shift);
+  const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
+  if (a.corr == SQUARED_DIFFERENCE) {
+    if (a.reduce == 0)
+      strip_backward_kernel<S, 0, 0><<<grid, block, smem, stream>>>(a, g);
+    else
+      strip_backward_kernel<S, 0, 1><<<grid, block, smem, stream>>>(a, g);
+  } else {
+    if (a.reduce == 0)
+      strip_backward_kernel<S, 1, 0><<<grid, block, smem, stream>>>(a, g);
+    else
+      strip_backward_kernel<S, 1, 1><<<grid, block, smem, stream>>>(a, g);
+  }
+  if ((err = hipGetLastError()) != hipSuccess) return err;
+  if constexpr (sizeof(S) == 2) {
+    if ((err = launch_narrow<S>(a.ref_grad_acc, a.ref_grad, n_ref, stream)) != hipSuccess) return err;
+    if ((err = launch_narrow<S>(a.src_grad_acc, a.src_grad, n_src, stream)) != hipSuccess) return err;
+  }
+  return hipSuccess;
+}
+
+#define CHOP_INSTANTIATE(S)                                                      \
+  template bool strip_supported<S>(const Args<S> &);                             \
+  template hipError_t launch_strip_forward<S>(const Args<S> &, hipStream_t);     \
+  template hipError_t launch_strip_backward<S>(const Args<S> &, hipStream_t);
+CHOP_INSTANTIATE(float)
+CHOP_INSTANTIATE(double)
+CHOP_INSTANTIATE(__half)
+CHOP_INSTANTIATE(bf16_t)
+#undef CHOP_INSTANTIATE
+
+}  // namespace chop

@@ -354,12 +354,14 @@ int chop_cost_volume_sample_coords_f64(void *stream, int half_centor, int64_t B,
                                        const double *Rs, const double *Ts, double *sw,
                                        double *sh, int32_t *fh, int32_t *fw, int32_t *state);
 
-/* Selects the kernel family for subsequent calls from this thread: 0 = automatic
- * (tiled kernels where the shape allows, otherwise the general kernels), 1 = general
- * kernels only.  Returns the previous value.  Used by the tests to cover both. */
+/* Selects the kernel family for subsequent calls from this thread: 0 = automatic (tiled
+ * kernels where the shape allows, otherwise the strip kernels, otherwise the general
+ * kernels), 1 = general kernels only, 2 = strip kernels where the shape allows (any storage
+ * type, up to 64 channels), otherwise the general kernels.  Returns the previous value.  Used
+ * by the tests to cover all three. */
 int chop_set_kernel_family(int family);
 /* Which family served the last forward/backward call of this thread: 0 none yet,
- * 1 general kernels, 2 tiled kernels. */
+ * 1 general kernels, 2 tiled kernels, 3 strip kernels. */
 int chop_last_kernel_family(void);
 
 #ifdef __cplusplus

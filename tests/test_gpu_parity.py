@@ -13,7 +13,7 @@ from gpu_util import (TORCH_DTYPE, assert_backward_close, assert_forward_close, 
 
 pytestmark = pytest.mark.gpu
 
-FAMILIES = [pytest.param(1, id="general"), pytest.param(0, id="auto")]
+FAMILIES = [pytest.param(1, id="general"), pytest.param(2, id="strip"), pytest.param(0, id="auto")]
 
 
 @pytest.fixture(autouse=True)
@@ -24,9 +24,12 @@ def _announce(request):
 
 
 def _assert_family(family, expect_tiled=True):
-    """Under the automatic selection the benchmark shapes must really run the tiled kernels."""
+    """Which kernels served the last call: 1 general, 2 tiled, 3 strip.  Under the automatic
+    selection the benchmark shapes must really run the tiled kernels; what those decline
+    (float64, channel counts other than 4 x 2^k) goes to the strip kernels."""
     got = _lib.load().chop_last_kernel_family()
-    assert got == (1 if family == 1 or not expect_tiled else 2), got
+    want = {1: 1, 2: 3, 0: 2 if expect_tiled else 3}[family]
+    assert got == want, (got, want)
 
 
 def _v1_inputs(t, dtype=None):
@@ -84,11 +87,10 @@ def test_v1_forward_reference_shapes(oracle, family, shape, reduce, dtype):
         t = reference_test_case(case, B, N, H, W, C, D, dtype, seed=case)
         want_cost, want_mask = oracle.cost_volume_fwd(**t, reduce=reduce)
         cost, mask = chop.cost_volume_raw(*_v1_inputs(t), reduce)
+        _assert_family(family, expect_tiled=False)  # C = 3 or 5: never the tiled kernels
         assert np.array_equal(host(mask), want_mask)
-        if family == 1:
-            assert np.array_equal(host(cost), want_cost)  # literal operation order: same bits
-        else:
-            assert_forward_close(host(cost), want_cost)
+        # general and strip kernels keep the literal operation order: same bits
+        assert np.array_equal(host(cost), want_cost)
 
 
 @pytest.mark.parametrize("family", FAMILIES)
@@ -145,6 +147,7 @@ def test_v1_backward_reference_shapes(oracle, family, shape, reduce, dtype):
         cg = rng.standard_normal((B, H, W, D, C)).astype(dtype)
         want = oracle.cost_volume_bwd(**t, cost_grad=cg, mask=mask, reduce=reduce)
         got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), dev(mask), reduce)
+        _assert_family(family, expect_tiled=False)
         tol = 1e-4 if dtype == np.float32 else 1e-10
         for g, w in zip(got, want):
             assert g.shape == w.shape
@@ -186,15 +189,14 @@ def test_v2_forward_backward_reference_shapes(oracle, family, reduce, dtype):
                                                              t["Ts"], reduce, 3)
             ins = [dev(t["ref"]), dev(t["src"]), dev(dg), dev(t["Rs"]), dev(t["Ts"])]
             cost, mask = chop.cost_volume_v2_raw(*ins, reduce, 3)
+            _assert_family(family, expect_tiled=False)  # C = 9
             assert np.array_equal(host(mask), want_mask)
-            if family == 1:
-                assert np.array_equal(host(cost), want_cost)
-            else:
-                assert_forward_close(host(cost), want_cost, atol=1e-5)
+            assert np.array_equal(host(cost), want_cost)
             cg = rng.standard_normal(want_cost.shape).astype(dtype)
             want = oracle.cost_volume_v2_bwd(t["ref"], t["src"], dg, t["Rs"], t["Ts"], cg,
                                              want_mask, reduce, 3)
             got = chop.cost_volume_grad_v2(*ins, dev(cg), dev(want_mask), reduce, 3)
+            _assert_family(family, expect_tiled=False)
             tol = 1e-4 if dtype == np.float32 else 1e-10
             for g, w in zip(got, want):
                 assert_backward_close(host(g), w, tol)
@@ -324,7 +326,7 @@ def test_backward_without_the_depth_gradient(oracle, family):
     acg = np.ascontiguousarray(t["cost_grad"][..., 0])
     want = oracle.cost_aggregate_bwd(*args, acg, amask)
     got = chop.cost_aggregate_grad(*_v1_inputs(t), dev(acg), dev(amask), need_depth_grad=False)
-    _assert_family(family)
+    _assert_family(1 if family == 2 else family)  # no strip kernels for CostAggregate
     assert got[2] is None
     assert_backward_close(host(got[0]), want[0])
     assert_backward_close(host(got[1]), want[1])
@@ -423,7 +425,7 @@ def test_golden_vectors(family):
             got = chop.cost_volume_grad_v2(*ins, dev(t["cost_grad"]), dev(want_mask), red_s, groups,
                                            bool(half))
         assert np.array_equal(host(mask), want_mask), name
-        if family == 1 or op >= 3:   # literal operation order: same bits
+        if family in (1, 2) or op >= 3:   # literal operation order: same bits
             assert np.array_equal(host(cost), want_cost), name
         else:
             assert_forward_close(host(cost), want_cost, atol=1e-5 if op == 1 else 1e-6)
