@@ -27,6 +27,8 @@ for _t in ("f32", "f64"):
     SIGNATURES["chop_cost_aggregate_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_vp] * 11
     SIGNATURES["chop_cost_volume_v2_fwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 7
     SIGNATURES["chop_cost_volume_v2_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 10
+    SIGNATURES["chop_cost_aggregate_fwd_fill_" + _t] = [_vp, _int, _int] + _DIMS + [_vp] * 9
+    SIGNATURES["chop_cost_volume_v2_fwd_fill_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 8
     SIGNATURES["chop_cost_volume_v3_fwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 8
     SIGNATURES["chop_cost_volume_v3_bwd_" + _t] = [_vp, _int, _int] + _DIMS + [_int] + [_vp] * 11
     SIGNATURES["chop_feature_aggregate_fwd_" + _t] = [_vp, _int] + _DIMS + [_vp] * 7
@@ -40,6 +42,7 @@ SIGNATURES["chop_cost_volume_bwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] 
 SIGNATURES["chop_cost_volume_bwd_16_static"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 12
 SIGNATURES["chop_static_scratch_bytes"] = []
 SIGNATURES["chop_cost_volume_v2_fwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 7
+SIGNATURES["chop_cost_volume_v2_fwd_fill_16"] = [_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 8
 SIGNATURES["chop_cost_volume_v2_bwd_16"] = ([_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 11
                                             + [ctypes.c_size_t])
 

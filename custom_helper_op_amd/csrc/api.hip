@@ -72,7 +72,8 @@ int forward(void *stream, int reduce, int half_centor, const Dims &d, int groups
             const S *ref, const S *src, const typename Storage<S>::Real *base_plane,
             const typename Storage<S>::Real *offsets, const typename Storage<S>::Real *depth_grid,
             const typename Storage<S>::Real *Rs, const typename Storage<S>::Real *Ts, S *cost,
-            int32_t *mask, bool needs_depth_grid) {
+            int32_t *mask, bool needs_depth_grid,
+            const typename Storage<S>::Real *default_cost = nullptr, bool needs_default = false) {
   using R = typename Storage<S>::Real;
   if (int rc = check_dims(d, reduce, groups, corr == GROUP_CORRELATION)) return rc;
   const int64_t pixels = d.B * d.H * d.W, voxels = pixels * d.D;
@@ -90,12 +91,14 @@ int forward(void *stream, int reduce, int half_centor, const Dims &d, int groups
   REQUIRE_PTR(Ts, d.B * d.N);
   REQUIRE_PTR(cost, voxels);
   REQUIRE_PTR(mask, voxels);
+  if (needs_default) REQUIRE_PTR(default_cost, voxels);
   Args<S> a{};
   a.B = d.B, a.H = d.H, a.W = d.W, a.C = d.C, a.D = d.D, a.N = d.N, a.srcH = d.srcH, a.srcW = d.srcW;
   a.groups = corr == GROUP_CORRELATION ? groups : 1;
   a.reduce = reduce, a.corr = corr, a.half = half_centor ? R(0.5) : R(0);
   a.ref = ref, a.src = src, a.base_plane = base_plane, a.offsets = offsets;
   a.depth_grid = depth_grid, a.Rs = Rs, a.Ts = Ts, a.cost = cost, a.mask = mask;
+  a.default_cost = default_cost;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (g_kernel_family == 0 && tiled_forward_supported(a)) {
     g_last_family = 2;
@@ -462,6 +465,33 @@ int chop_cost_volume_v2_bwd_f64(void *stream, int reduce, int half_centor, int64
                           src_grad, depth_grid_grad, true, nullptr, 0);
 }
 
+// The forward ops of the two cost-map layers with the layers' default fill folded into the
+// store (custom_helper_op/python/layers/custom_layers.py:51-57, :77-83).
+#define FILL_ENTRY(SFX, T)                                                                      \
+  int chop_cost_aggregate_fwd_fill_##SFX(void *stream, int reduce, int half_centor, int64_t B,  \
+                                         int64_t H, int64_t W, int64_t C, int64_t D, int64_t N, \
+                                         int64_t srcH, int64_t srcW, const T *ref, const T *src, \
+                                         const T *base_plane, const T *offsets, const T *Rs,    \
+                                         const T *Ts, const T *default_cost, T *cost,           \
+                                         int32_t *mask) {                                       \
+    return forward<T>(stream, reduce, half_centor, DIMS, 1, SUM_SQUARED_DIFFERENCE, ref, src,   \
+                      base_plane, offsets, nullptr, Rs, Ts, cost, mask, false, default_cost,    \
+                      true);                                                                    \
+  }                                                                                             \
+  int chop_cost_volume_v2_fwd_fill_##SFX(void *stream, int reduce, int half_centor, int64_t B,  \
+                                         int64_t H, int64_t W, int64_t C, int64_t D, int64_t N, \
+                                         int64_t srcH, int64_t srcW, int groups, const T *ref,  \
+                                         const T *src, const T *depth_grid, const T *Rs,        \
+                                         const T *Ts, const T *default_cost, T *cost,           \
+                                         int32_t *mask) {                                       \
+    return forward<T>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION, ref, src,   \
+                      nullptr, nullptr, depth_grid, Rs, Ts, cost, mask, true, default_cost,     \
+                      true);                                                                    \
+  }
+FILL_ENTRY(f32, float)
+FILL_ENTRY(f64, double)
+#undef FILL_ENTRY
+
 #define V3_ENTRY(SFX, T)                                                                       \
   int chop_cost_volume_v3_fwd_##SFX(void *stream, int reduce, int half_centor, int64_t B,      \
                                     int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,     \
@@ -536,7 +566,6 @@ V3_ENTRY(f64, double)
     REQUIRE_PTR(default_grad, 1);                                                               \
     REQUIRE_PTR(out_grad, total);                                                               \
     REQUIRE_PTR(mask, total);                                                                   \
-    REQUIRE_PTR(cost_grad, total);                                                              \
     return launch_status(launch_default_fill_grad<T>(reduce, mask_count, inner, out_grad, mask, \
                                                      cost_grad, default_grad,                   \
                                                      static_cast<hipStream_t>(stream)),         \
@@ -654,6 +683,21 @@ int chop_cost_volume_v2_fwd_16(void *stream, int storage, int reduce, int half_c
       forward<bf16_t>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
                       (const bf16_t *)ref, (const bf16_t *)src, nullptr, nullptr, depth_grid, Rs,
                       Ts, (bf16_t *)cost, mask, true))
+}
+
+int chop_cost_volume_v2_fwd_fill_16(void *stream, int storage, int reduce, int half_centor,
+                                    int64_t B, int64_t H, int64_t W, int64_t C, int64_t D,
+                                    int64_t N, int64_t srcH, int64_t srcW, int groups,
+                                    const void *ref, const void *src, const float *depth_grid,
+                                    const float *Rs, const float *Ts, const float *default_cost,
+                                    void *cost, int32_t *mask) {
+  STORAGE_DISPATCH(
+      forward<__half>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
+                      (const __half *)ref, (const __half *)src, nullptr, nullptr, depth_grid, Rs,
+                      Ts, (__half *)cost, mask, true, default_cost, true),
+      forward<bf16_t>(stream, reduce, half_centor, DIMS, groups, GROUP_CORRELATION,
+                      (const bf16_t *)ref, (const bf16_t *)src, nullptr, nullptr, depth_grid, Rs,
+                      Ts, (bf16_t *)cost, mask, true, default_cost, true))
 }
 
 int chop_cost_volume_v2_bwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kBlock) void default_fill_grad_kernel(int reduce, i
     const int32_t m = mask[e / inner];
     const bool keep = reduce == 0 ? m > 0 : m >= 0;
     const R g = out_grad[e];
-    cost_grad[e] = keep ? g : R(0);
+    if (cost_grad != nullptr) cost_grad[e] = keep ? g : R(0);
     if (!keep) sum += g;
   }
   // wavefront sum, then one atomic per workgroup

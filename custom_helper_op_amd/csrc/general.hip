@@ -70,6 +70,7 @@ __global__ __launch_bounds__(kBlock) void general_forward_kernel(const Args<S> a
     } else {
       a.mask[e] = arg;
     }
+    if (a.default_cost != nullptr && (REDUCE == 0 ? used == 0 : arg < 0)) acc = *a.default_cost;
     Storage<S>::store(a.cost + e, acc);
   }
 }
@@ -117,6 +118,7 @@ __global__ __launch_bounds__(kBlock) void general_aggregate_forward_kernel(const
     } else if (used >= 0) {
       out = acc / static_cast<R>(C);
     }
+    if (a.default_cost != nullptr && (REDUCE == 0 ? used <= 0 : used < 0)) out = *a.default_cost;
     Storage<S>::store(a.cost + i, out);
   }
 }

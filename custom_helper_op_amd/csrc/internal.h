@@ -45,6 +45,10 @@ struct Args {
   // forward
   S *cost;
   int32_t *mask;
+  // forward, optional (device scalar): stored instead of the cost wherever no view was
+  // accepted (MEAN: count 0, MIN: winner -1) -- the cost-map layers' default fill
+  // (custom_helper_op/python/layers/custom_layers.py:52-57, :78-83) folded into the store
+  const R *default_cost;
   // backward
   const S *cost_grad;
   const int32_t *mask_in;

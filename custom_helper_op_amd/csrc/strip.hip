@@ -116,6 +116,8 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
   const bool ch_ok = cl < C, out_ok = px.ok && cl < OC;
   const R ref_c = ch_ok ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
+  const bool fill = a.default_cost != nullptr;  // the cost-map layers' default for empty voxels
+  const R dflt = fill ? *a.default_cost : R(0);
   const int64_t row_step = (int64_t)srcW * C;
   StripRecords<R> rec = strip_records<R, 4>(smem, ppw);
   R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw)) - 64;  // CORR: products of a pixel
@@ -199,6 +201,7 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
       } else if (out_ok) {
         a.mask[i * OC + cl] = arg[jj];
       }
+      if (fill && (REDUCE == 0 ? kcnt[jj] == 0 : arg[jj] < 0)) acc[jj] = dflt;
       if (out_ok) Storage<S>::store(a.cost + i * OC + cl, acc[jj]);
     }
   }

@@ -46,6 +46,8 @@ struct Geometry {
   int64_t units_per_xcd;   // ceil(total_units / 8)
   int xcd_shift;           // log2 of the units dealt to one XCD at a time; -1: one band per XCD
   int64_t grid;            // workgroups to launch
+  int tile_cols;           // pixels per tile row: PPW (one row of pixels) or PPW/2 (two rows)
+  int tiles_x;             // two-row tiles per image row
   int sub;                 // channels per correlation group (1 for squared difference)
   float src_h_max, src_w_max;  // (float)(srcH - 1), (float)(srcW - 1): acceptance bounds
 };
@@ -277,7 +279,16 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
   const int t_in = (int)(tile - (unsigned)t.b * (unsigned)g.tiles_per_image);
   t.p = t.lane / LPP;
   t.cl = t.lane % LPP;
-  t.pin = t_in * PPW + t.p;
+  if (g.tile_cols == PPW) {
+    t.pin = t_in * PPW + t.p;
+  } else {
+    // two rows of PPW/2 pixels: the samples of a compact tile cross texel boundaries at more
+    // nearly the same depths than those of a long row, so fewer wave iterations carry a
+    // cell change (0.49 against 0.62 of them on the MVSNet-stage workload)
+    const int ty = t_in / g.tiles_x, tx = t_in - ty * g.tiles_x;
+    const int py = t.p >= g.tile_cols ? 1 : 0;
+    t.pin = (ty * 2 + py) * (int)a.W + tx * g.tile_cols + (t.p - py * g.tile_cols);
+  }
   t.pix_ok = t.pin < g.hw;
   if (!t.pix_ok) t.pin = g.hw - 1;  // clamp: loads stay in range, stores are predicated
   t.pix = (int64_t)t.b * g.hw + t.pin;
@@ -539,6 +550,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
   const int OC = CORR == 1 ? a.groups : (CORR == 2 || CORR == 3) ? 1 : C;
   const int gv = VEC / g.sub;  // output values per lane
   const int d_lo = t.d_lo, d_hi = t.d_hi;
+  // the cost-map layers' default fill folded into the store: where no view was accepted the
+  // scalar is written instead of the cost (custom_layers.py:52-57, :78-83)
+  const bool fill = a.default_cost != nullptr;
+  const float dflt = fill ? *a.default_cost : 0.f;
   // this pixel's output rows (the 64-bit product once per wave, not once per depth)
   S *const out_pix = a.cost + t.pix * D * OC;
   int32_t *const mask_pix = a.mask + t.pix * D * OC;
@@ -655,7 +670,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       }
       const int d = d0 + t.cl;
       if (d < d_hi && t.pix_ok) {
-        const float out = win >= 0 ? best / static_cast<float>(C) : 0.f;  // :222-227
+        const float out = win >= 0 ? best / static_cast<float>(C) : dflt;  // :222-227
         __builtin_nontemporal_store(out, reinterpret_cast<float *>(a.cost) + t.pix * D + d);
         __builtin_nontemporal_store(win, a.mask + t.pix * D + d);
       }
@@ -768,6 +783,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
         if constexpr (REDUCE == 1) {
           int32_t *mout = mask_pix + d * OC;
+          if (fill) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c)
+              if (arg[jj][c] < 0) acc[jj][c] = dflt;
+          }
           if (CORR == 0) {
             store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
             store_ints<VEC>(mout + t.cl * VEC, arg[jj]);
@@ -784,10 +804,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
             for (int c = 0; c < VEC; ++c) acc[jj][c] *= inv;
           }
           if (CORR == 0) {
+            if (fill && kcnt[jj] == 0) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) acc[jj][c] = dflt;
+            }
             store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
           } else {
             float grp[VEC];
             fold_groups<VEC>(acc[jj], g.sub, grp);
+            if (fill && kcnt[jj] == 0) {
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) grp[c] = dflt;
+            }
             store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
           }
         }
@@ -965,6 +993,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         continue;
       }
       if constexpr (REDUCE == 1) {
+        if (fill) {
+#pragma unroll
+          for (int c = 0; c < VEC; ++c)
+            if (arg[c] < 0) acc[c] = dflt;
+        }
         if (t.pix_ok) {
           S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
           int32_t *mout = mask_pix + d * OC;
@@ -985,7 +1018,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
         // slice index equals the depth's place in the chunk keeps the result, so that the
         // chunk is stored as LPP consecutive floats per pixel
         float tot = group_sum<LPP>((acc[0] + acc[1]) + (acc[2] + acc[3]));
-        tot = k > 0 ? tot / static_cast<float>(k * C) : 0.f;
+        tot = k > 0 ? tot / static_cast<float>(k * C) : dflt;
         if constexpr (LPP > 1) {
           if (t.cl == jj) agg_out = tot;
         } else {
@@ -1001,10 +1034,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
       if (t.pix_ok) {
         S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
         if (CORR == 0) {
+          if (fill && k == 0) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) acc[c] = dflt;
+          }
           store_vec<S, VEC, true>(out + t.cl * VEC, acc);
         } else {
           float grp[VEC];
           fold_groups<VEC>(acc, g.sub, grp);
+          if (fill && k == 0) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) grp[c] = dflt;
+          }
           store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
         }
       }
@@ -1603,9 +1644,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
     for (int jj = 0; jj < LPP; ++jj) {
       const int d = d0 + jj;
-      if (d >= d_hi) {
-        if constexpr (LPP >= 16) continue; else break;  // see the forward kernel
-      }
+      // (no early exit past d_hi: the records of such depths carry a zero factor and no tap
+      // offset, the row loads are clamped, and a loop without exits compiles to faster code)
       if constexpr (LPP > PF && !kVoxelGrad) {
         if (jj > 0 && jj % PF == 0) load_rows(d0 + jj);  // next part of a deep chunk
       }
@@ -1851,6 +1891,13 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   Geometry g;
   g.hw = (int)(H * W);
   g.tiles_per_image = (g.hw + PPW - 1) / PPW;
+  // two-row tiles where they tile the image exactly
+  g.tile_cols = PPW;
+  g.tiles_x = 1;
+  if (PPW >= 2 && H % 2 == 0 && W % (PPW / 2) == 0) {
+    g.tile_cols = PPW / 2;
+    g.tiles_x = (int)(W / (PPW / 2));
+  }
   const int64_t tiles = B * g.tiles_per_image;
   g.ngroups = ngroups;
   g.vper = vper;

@@ -1,8 +1,9 @@
 """The reference's cost-map layers on top of the operators
 (custom_helper_op/python/layers/custom_layers.py:33-84), as torch modules.
 
-``CostMapLayer`` runs CostAggregate and ``CostMapLayerV2`` runs CostVolumeV2; both then replace
-the cost of every voxel that no source view covered by a scalar ``default_cost``.
+``CostMapLayer`` runs CostAggregate and ``CostMapLayerV2`` runs CostVolumeV2; both replace the
+cost of every voxel that no source view covered by a scalar ``default_cost`` -- here inside
+the op's own store, so the forward is one kernel.
 ``default_type`` keeps the reference's meaning: ``'DYNAMIC'`` a trainable scalar initialised to
 zero, ``'CONSTANT'`` the same scalar but frozen, a tensor (V2) or number the fixed value itself.
 """
@@ -26,9 +27,8 @@ class _CostMapBase(torch.nn.Module):
         else:
             self.register_buffer("default_cost", torch.as_tensor(default_type, dtype=torch.float32))
 
-    def _fill(self, cost, cost_mask):
-        default = self.default_cost.to(device=cost.device, dtype=cost.dtype)
-        return ops.cost_default_fill(cost, cost_mask, default, self.reduce_method)
+    def _default(self, like, real_dtype):
+        return self.default_cost.to(device=like.device, dtype=real_dtype)
 
 
 class CostMapLayer(_CostMapBase):
@@ -39,9 +39,10 @@ class CostMapLayer(_CostMapBase):
         super().__init__(reduce_method, half_centor, default_type)
 
     def forward(self, inputs):
-        cost, cost_mask = ops.cost_aggregate(*inputs, reduce_method=self.reduce_method,
-                                             half_centor=self.half_centor)
-        return self._fill(cost, cost_mask), cost_mask
+        ref = inputs[0]
+        return ops.cost_aggregate_filled(*inputs, self._default(ref, ref.dtype),
+                                         reduce_method=self.reduce_method,
+                                         half_centor=self.half_centor)
 
 
 class CostMapLayerV2(_CostMapBase):
@@ -53,6 +54,8 @@ class CostMapLayerV2(_CostMapBase):
         self.groups = groups
 
     def forward(self, inputs):
-        cost, cost_mask = ops.cost_volume_v2(*inputs, reduce_method=self.reduce_method,
-                                             groups=self.groups, half_centor=self.half_centor)
-        return self._fill(cost, cost_mask), cost_mask
+        ref = inputs[0]
+        real = torch.float32 if ref.dtype in (torch.float16, torch.bfloat16) else ref.dtype
+        return ops.cost_volume_v2_filled(*inputs, self._default(ref, real),
+                                         reduce_method=self.reduce_method, groups=self.groups,
+                                         half_centor=self.half_centor)

@@ -192,8 +192,16 @@ def cost_volume_grad(ref_image, src_images, base_plane, offsets, rs, ts, cost_gr
     return ref_grad, src_grad, bp_grad
 
 
+def _prep_default(default_cost, rdt, dev):
+    default_cost = _prep(default_cost, rdt, dev, "default_cost")
+    _require(default_cost.numel() == 1, "default_cost must be a scalar")
+    return default_cost
+
+
 def cost_volume_v2_raw(ref_image, src_images, depth_grid, Rs, Ts, reduce_method="MEAN", groups=None,
-                       half_centor=True):
+                       half_centor=True, default_cost=None):
+    """``default_cost`` (a device scalar): written instead of the cost wherever no view was
+    accepted -- ``CostMapLayerV2``'s fill, done by the op's own store."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
@@ -206,7 +214,20 @@ def cost_volume_v2_raw(ref_image, src_images, depth_grid, Rs, Ts, reduce_method=
     cost = torch.empty((B, H, W, D, groups), dtype=dt, device=dev)
     mask = torch.empty((B, H, W, D, 1 if red == 0 else groups), dtype=torch.int32, device=dev)
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
-    if dt in _STORAGE16:
+    if default_cost is not None:
+        default_cost = _prep_default(default_cost, rdt, dev)
+        if dt in _STORAGE16:
+            rc = lib.chop_cost_volume_v2_fwd_fill_16(
+                _stream(cost), _STORAGE16[dt], red, int(half_centor), *dims, groups,
+                _ptr(ref_image), _ptr(src_images), _ptr(depth_grid), _ptr(Rs), _ptr(Ts),
+                _ptr(default_cost), _ptr(cost), _ptr(mask))
+        else:
+            fn = (lib.chop_cost_volume_v2_fwd_fill_f32 if dt == torch.float32
+                  else lib.chop_cost_volume_v2_fwd_fill_f64)
+            rc = fn(_stream(cost), red, int(half_centor), *dims, groups, _ptr(ref_image),
+                    _ptr(src_images), _ptr(depth_grid), _ptr(Rs), _ptr(Ts), _ptr(default_cost),
+                    _ptr(cost), _ptr(mask))
+    elif dt in _STORAGE16:
         rc = lib.chop_cost_volume_v2_fwd_16(_stream(cost), _STORAGE16[dt], red, int(half_centor),
                                             *dims, groups, _ptr(ref_image), _ptr(src_images),
                                             _ptr(depth_grid), _ptr(Rs), _ptr(Ts), _ptr(cost),
@@ -263,10 +284,11 @@ def cost_volume_grad_v2(ref_image, src_images, depth_grid, rs, ts, cost_grad, co
 
 
 def cost_aggregate_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduce_method="MEAN",
-                       half_centor=True):
+                       half_centor=True, default_cost=None):
     """The ``CostAggregate`` op without autograd: ``(cost [B,H,W,D], cost_mask int32 [B,H,W,D])``
     (shapes: custom_helper_op/cc/ops/custom_helper_ops.cc:46-58; checks:
-    cost_aggregate_kernels.cc:85-106).  float32 and float64 only, as registered."""
+    cost_aggregate_kernels.cc:85-106).  float32 and float64 only, as registered.
+    ``default_cost`` as in :func:`cost_volume_v2_raw` (``CostMapLayer``'s fill)."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     dt, dev = ref_image.dtype, ref_image.device
@@ -280,9 +302,17 @@ def cost_aggregate_raw(ref_image, src_images, base_plane, offsets, Rs, Ts, reduc
     cost = torch.empty((B, H, W, D), dtype=dt, device=dev)
     mask = torch.empty((B, H, W, D), dtype=torch.int32, device=dev)
     dims = (B, H, W, C, D, N, src_images.shape[2], src_images.shape[3])
-    fn = lib.chop_cost_aggregate_fwd_f32 if dt == torch.float32 else lib.chop_cost_aggregate_fwd_f64
-    rc = fn(_stream(cost), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
-            _ptr(base_plane), _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(cost), _ptr(mask))
+    if default_cost is not None:
+        default_cost = _prep_default(default_cost, dt, dev)
+        fn = (lib.chop_cost_aggregate_fwd_fill_f32 if dt == torch.float32
+              else lib.chop_cost_aggregate_fwd_fill_f64)
+        rc = fn(_stream(cost), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
+                _ptr(base_plane), _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(default_cost), _ptr(cost),
+                _ptr(mask))
+    else:
+        fn = lib.chop_cost_aggregate_fwd_f32 if dt == torch.float32 else lib.chop_cost_aggregate_fwd_f64
+        rc = fn(_stream(cost), red, int(half_centor), *dims, _ptr(ref_image), _ptr(src_images),
+                _ptr(base_plane), _ptr(offsets), _ptr(Rs), _ptr(Ts), _ptr(cost), _ptr(mask))
     _lib.check(rc)
     return cost, mask
 
@@ -517,6 +547,88 @@ class _CostAggregate(torch.autograd.Function):
                                          grad_out.contiguous(), mask, *ctx.attrs,
                                          need_depth_grad=ctx.needs_input_grad[2])
         return rg, sg, bg, None, None, None, None, None
+
+
+def _default_grad(grad_out, mask, reduce_method, like):
+    """Gradient of the layers' scalar default: the upstream gradient summed over the voxels
+    that received it (one reduction kernel; the 16-bit storage types are widened first)."""
+    lib = _lib.load()
+    red = _reduce_code(reduce_method)
+    g = grad_out.contiguous()
+    if g.dtype in _STORAGE16:
+        g = g.float()
+    n_mask = mask.numel()
+    inner = g.numel() // n_mask if n_mask else 1
+    out = torch.empty((), dtype=g.dtype, device=g.device)
+    fn = (lib.chop_cost_default_fill_grad_f32 if g.dtype == torch.float32
+          else lib.chop_cost_default_fill_grad_f64)
+    _lib.check(fn(_stream(out), red, n_mask, inner, _ptr(g), _ptr(mask), None, _ptr(out)))
+    return out.to(like.dtype).reshape(like.shape)
+
+
+class _CostVolumeV2Filled(torch.autograd.Function):
+    """``CostMapLayerV2.call`` (custom_layers.py:77-83) as one forward kernel: CostVolumeV2 whose
+    store writes ``default_cost`` where no view was accepted.  The op's registered gradient
+    skips exactly those voxels, so it takes the upstream gradient as it is."""
+
+    @staticmethod
+    def forward(ctx, ref_image, src_images, depth_grid, Rs, Ts, default_cost, reduce_method, groups,
+                half_centor):
+        cost, mask = cost_volume_v2_raw(ref_image, src_images, depth_grid, Rs, Ts, reduce_method,
+                                        groups, half_centor, default_cost=default_cost)
+        ctx.save_for_backward(ref_image, src_images, depth_grid, Rs, Ts, mask, default_cost)
+        ctx.attrs = (reduce_method, groups, half_centor)
+        ctx.mark_non_differentiable(mask)
+        return cost, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        ref_image, src_images, depth_grid, Rs, Ts, mask, default_cost = ctx.saved_tensors
+        rg, sg, dg = cost_volume_grad_v2(ref_image, src_images, depth_grid, Rs, Ts,
+                                         grad_out.contiguous(), mask, *ctx.attrs,
+                                         need_depth_grad=ctx.needs_input_grad[2])
+        dd = (_default_grad(grad_out, mask, ctx.attrs[0], default_cost)
+              if ctx.needs_input_grad[5] else None)
+        return rg, sg, dg, None, None, dd, None, None, None
+
+
+class _CostAggregateFilled(torch.autograd.Function):
+    """``CostMapLayer.call`` (custom_layers.py:51-57) as one forward kernel."""
+
+    @staticmethod
+    def forward(ctx, ref_image, src_images, base_plane, offsets, Rs, Ts, default_cost, reduce_method,
+                half_centor):
+        cost, mask = cost_aggregate_raw(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                        reduce_method, half_centor, default_cost=default_cost)
+        ctx.save_for_backward(ref_image, src_images, base_plane, offsets, Rs, Ts, mask, default_cost)
+        ctx.attrs = (reduce_method, half_centor)
+        ctx.mark_non_differentiable(mask)
+        return cost, mask
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_mask):
+        ref_image, src_images, base_plane, offsets, Rs, Ts, mask, default_cost = ctx.saved_tensors
+        rg, sg, bg = cost_aggregate_grad(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                         grad_out.contiguous(), mask, *ctx.attrs,
+                                         need_depth_grad=ctx.needs_input_grad[2])
+        dd = (_default_grad(grad_out, mask, ctx.attrs[0], default_cost)
+              if ctx.needs_input_grad[6] else None)
+        return rg, sg, bg, None, None, None, dd, None, None
+
+
+def cost_volume_v2_filled(ref_image, src_images, depth_grid, Rs, Ts, default_cost,
+                          reduce_method="MEAN", groups=None, half_centor=True):
+    """CostVolumeV2 followed by ``where(valid(cost_mask), cost, default_cost)``, fused into one
+    kernel; differentiable in the images, the depth grid and the scalar."""
+    return _CostVolumeV2Filled.apply(ref_image, src_images, depth_grid, Rs, Ts, default_cost,
+                                     reduce_method, groups, half_centor)
+
+
+def cost_aggregate_filled(ref_image, src_images, base_plane, offsets, Rs, Ts, default_cost,
+                          reduce_method="MEAN", half_centor=True):
+    """CostAggregate followed by the same fill, fused into one kernel."""
+    return _CostAggregateFilled.apply(ref_image, src_images, base_plane, offsets, Rs, Ts,
+                                      default_cost, reduce_method, half_centor)
 
 
 class _CostVolumeV3(torch.autograd.Function):

@@ -249,7 +249,8 @@ int chop_feature_aggregate_bwd_f64(void *stream, int half_centor, int64_t B, int
  * elements, `inner` consecutive ones per mask entry (CostAggregate: inner 1, mask [B,H,W,D];
  * CostVolumeV2 MEAN: inner = groups, mask [B,H,W,D,1]; CostVolumeV2 MIN: inner 1, mask
  * [B,H,W,D,groups]).  out may be the cost buffer itself.
- * The gradient of that `where`: cost_grad = out_grad where valid and 0 elsewhere,
+ * The gradient of that `where`: cost_grad = out_grad where valid and 0 elsewhere (cost_grad
+ * may be NULL when only the scalar's gradient is wanted),
  * *default_grad = sum of out_grad where not valid (the entry zeroes it first). */
 int chop_cost_default_fill_f32(void *stream, int reduce, int64_t mask_count, int64_t inner,
                                const float *cost, const int32_t *mask, const float *default_cost,
@@ -274,6 +275,38 @@ int chop_combine_projection_f32(void *stream, int64_t B, int64_t N, const float 
 int chop_combine_projection_f64(void *stream, int64_t B, int64_t N, const double *ref_cam,
                                 const double *src_cam, const double *scale, double *Rs,
                                 double *Ts);
+
+/* The two layers' forward as one call: CostAggregate (CostMapLayer,
+ * custom_layers.py:51-57) and CostVolumeV2 (CostMapLayerV2, :77-83) with that default fill
+ * folded into the kernels' store, so the cost volume is written once instead of being read
+ * back and rewritten.  `default_cost` is the layer's device scalar; cost and mask are what
+ * chop_cost_aggregate_fwd_* / chop_cost_volume_v2_fwd_* followed by chop_cost_default_fill_*
+ * produce, bit for bit.  The gradients are those of the plain ops (voxels that received the
+ * default take no gradient there either) plus chop_cost_default_fill_grad_* for the scalar. */
+int chop_cost_aggregate_fwd_fill_f32(void *stream, int reduce, int half_centor, int64_t B,
+                                     int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                                     int64_t srcH, int64_t srcW, const float *ref,
+                                     const float *src, const float *base_plane,
+                                     const float *offsets, const float *Rs, const float *Ts,
+                                     const float *default_cost, float *cost, int32_t *mask);
+int chop_cost_aggregate_fwd_fill_f64(void *stream, int reduce, int half_centor, int64_t B,
+                                     int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                                     int64_t srcH, int64_t srcW, const double *ref,
+                                     const double *src, const double *base_plane,
+                                     const double *offsets, const double *Rs, const double *Ts,
+                                     const double *default_cost, double *cost, int32_t *mask);
+int chop_cost_volume_v2_fwd_fill_f32(void *stream, int reduce, int half_centor, int64_t B,
+                                     int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                                     int64_t srcH, int64_t srcW, int groups, const float *ref,
+                                     const float *src, const float *depth_grid, const float *Rs,
+                                     const float *Ts, const float *default_cost, float *cost,
+                                     int32_t *mask);
+int chop_cost_volume_v2_fwd_fill_f64(void *stream, int reduce, int half_centor, int64_t B,
+                                     int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
+                                     int64_t srcH, int64_t srcW, int groups, const double *ref,
+                                     const double *src, const double *depth_grid,
+                                     const double *Rs, const double *Ts,
+                                     const double *default_cost, double *cost, int32_t *mask);
 
 /* ---- 16-bit storage extension --------------------------------------------------------
  * No counterpart in the reference, whose ops register float32 and float64 only
@@ -325,6 +358,12 @@ int chop_cost_volume_v2_fwd_16(void *stream, int storage, int reduce, int half_c
                                int64_t srcH, int64_t srcW, int groups, const void *ref,
                                const void *src, const float *depth_grid, const float *Rs,
                                const float *Ts, void *cost, int32_t *mask);
+int chop_cost_volume_v2_fwd_fill_16(void *stream, int storage, int reduce, int half_centor,
+                                    int64_t B, int64_t H, int64_t W, int64_t C, int64_t D,
+                                    int64_t N, int64_t srcH, int64_t srcW, int groups,
+                                    const void *ref, const void *src, const float *depth_grid,
+                                    const float *Rs, const float *Ts, const float *default_cost,
+                                    void *cost, int32_t *mask);
 int chop_cost_volume_v2_bwd_16(void *stream, int storage, int reduce, int half_centor, int64_t B,
                                int64_t H, int64_t W, int64_t C, int64_t D, int64_t N,
                                int64_t srcH, int64_t srcW, int groups, const void *ref,

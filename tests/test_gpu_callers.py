@@ -107,3 +107,72 @@ def test_cost_map_layers(oracle, reduce):
     assert np.array_equal(host(mask2), want_mask2)
     want2 = oracle.cost_default_fill(want_cost2, want_mask2, np.float32(1.5), reduce)
     np.testing.assert_allclose(host(cost2), want2, rtol=1e-5, atol=1e-5)
+
+
+FAMILIES = [pytest.param(1, id="general"), pytest.param(2, id="strip"), pytest.param(0, id="auto")]
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_fill_folded_into_the_forward(oracle, family, reduce, dtype):
+    """The ops with a default_cost write, in one kernel, exactly what the plain op followed by
+    the layers' `where` gives: the op's own output with the default selected in, bit for bit
+    (every kernel family; CostAggregate and CostVolumeV2, which the two layers run)."""
+    lib = _lib.load()
+    lib.chop_set_kernel_family(family)
+    try:
+        t = reference_test_case(3, 2, 2, 20, 24, 8, 9, dtype, seed=6)
+        t["Ts"][:, 1, 2] = -40.0                       # the second view sees nothing
+        t["Ts"][0, 0, 0] = 400.0                       # and the first one nothing of batch item 0
+        keys = ("ref", "src", "base_plane", "offsets", "Rs", "Ts")
+        td = getattr(torch, np.dtype(dtype).name)
+        default = torch.tensor(-0.625, dtype=td, device="cuda")
+        ins = [dev(t[k]) for k in keys]
+        plain, mask = chop.cost_aggregate_raw(*ins, reduce)
+        fam_plain = lib.chop_last_kernel_family()
+        filled, mask_f = chop.cost_aggregate_raw(*ins, reduce, default_cost=default)
+        assert lib.chop_last_kernel_family() == fam_plain
+        assert np.array_equal(host(mask_f), host(mask))
+        want = oracle.cost_default_fill(host(plain), host(mask), dtype(-0.625), reduce)
+        assert np.array_equal(host(filled), want)
+        empty = (host(mask) <= 0) if reduce == "MEAN" else (host(mask) < 0)
+        assert empty.any() and not empty.all()
+
+        grid = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(dtype)
+        ins2 = [dev(t["ref"]), dev(t["src"]), dev(grid), dev(t["Rs"]), dev(t["Ts"])]
+        for groups in (4, 8, 1):
+            plain, mask = chop.cost_volume_v2_raw(*ins2, reduce, groups)
+            fam_plain = lib.chop_last_kernel_family()
+            filled, mask_f = chop.cost_volume_v2_raw(*ins2, reduce, groups, default_cost=default)
+            assert lib.chop_last_kernel_family() == fam_plain
+            assert np.array_equal(host(mask_f), host(mask))
+            want = oracle.cost_default_fill(host(plain), host(mask), dtype(-0.625), reduce)
+            assert np.array_equal(host(filled), want), groups
+    finally:
+        lib.chop_set_kernel_family(0)
+
+
+@pytest.mark.parametrize("storage", [torch.float16, torch.bfloat16])
+def test_cost_map_layer_v2_16bit(oracle, storage):
+    """CostMapLayerV2 on 16-bit features (the op beneath it supports them): forward against the
+    float32 oracle on the quantised inputs, and the scalar's gradient."""
+    from custom_helper_op_amd.configs import quantise
+    name = "f16" if storage == torch.float16 else "bf16"
+    t = reference_test_case(3, 1, 2, 16, 24, 8, 6, np.float32, seed=9)
+    t["Ts"][:, 1, 2] = -40.0
+    ref, src = quantise(t["ref"] * 0.1, name), quantise(t["src"] * 0.1, name)
+    grid = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(np.float32)
+    layer = chop.CostMapLayerV2(reduce_method="MEAN", groups=4, default_type="DYNAMIC").cuda()
+    with torch.no_grad():
+        layer.default_cost.fill_(0.5)
+    cost, mask = layer([dev(ref, storage), dev(src, storage), dev(grid), dev(t["Rs"]), dev(t["Ts"])])
+    assert cost.dtype == storage
+    want_cost, want_mask = oracle.cost_volume_v2_fwd(ref, src, grid, t["Rs"], t["Ts"], "MEAN", 4)
+    assert np.array_equal(host(mask), want_mask)
+    want = oracle.cost_default_fill(want_cost, want_mask, np.float32(0.5), "MEAN")
+    np.testing.assert_allclose(host(cost), want, rtol=1e-2, atol=1e-2)
+    empty = want_mask <= 0
+    assert empty.any() and not empty.all()
+    cost.float().sum().backward()
+    assert float(layer.default_cost.grad) == pytest.approx(float(empty.sum()) * 4, rel=1e-3)
