@@ -1356,7 +1356,11 @@ constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 :
 // DG: false when the caller does not want the depth gradient (a NULL output): the four
 // depth-derivative weights per record and the 20 instructions per wave-iteration that use
 // them drop out.
-template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true>
+// PV: the depth hypotheses come from a per-voxel depth_grid (and the depth gradient is per
+// voxel); a compile-time flag, because the kernel without the unused variant's code is
+// measurably faster than one that tests a.depth_grid at run time.
+template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true,
+          bool PV = (CORR == 1)>
 __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
   using WN = Window<VEC, LPP>;
@@ -1367,7 +1371,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   if (!locate_tile<S, LPP>(a, g, t)) return;
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
   const float half = a.half;
-  const bool per_voxel_depth = a.depth_grid != nullptr;
+  constexpr bool per_voxel_depth = PV;
   // byte offsets of the record arrays; a record is addressed as (lane-dependent byte offset)
   // + (compile-time constant), so that the constant lands in the instruction's offset field
   constexpr int kWts = 0, kDwt = kWts + NV * 64 * 16, kCell = kDwt + NV * 64 * 16,
