@@ -46,8 +46,7 @@ struct Geometry {
   int64_t units_per_xcd;   // ceil(total_units / 8)
   int xcd_shift;           // log2 of the units dealt to one XCD at a time; -1: one band per XCD
   int64_t grid;            // workgroups to launch
-  int tile_cols;           // pixels per tile row: PPW (one row of pixels) or PPW/2 (two rows)
-  int tiles_x;             // two-row tiles per image row
+  int tiles_x;             // tiles per image row (a tile: two rows of PPW/2 pixels)
   int sub;                 // channels per correlation group (1 for squared difference)
   float src_h_max, src_w_max;  // (float)(srcH - 1), (float)(srcW - 1): acceptance bounds
 };
@@ -279,17 +278,21 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
   const int t_in = (int)(tile - (unsigned)t.b * (unsigned)g.tiles_per_image);
   t.p = t.lane / LPP;
   t.cl = t.lane % LPP;
-  if (g.tile_cols == PPW) {
-    t.pin = t_in * PPW + t.p;
+  if constexpr (PPW == 1) {
+    t.pin = t_in;
+    t.pix_ok = true;
   } else {
-    // two rows of PPW/2 pixels: the samples of a compact tile cross texel boundaries at more
-    // nearly the same depths than those of a long row, so fewer wave iterations carry a
-    // cell change (0.49 against 0.62 of them on the MVSNet-stage workload)
+    // A tile is two rows of PPW/2 pixels: the samples of a compact tile cross texel boundaries
+    // at more nearly the same depths than those of a long row, so fewer wave iterations carry
+    // a cell change (0.49 against 0.62 of them on the MVSNet-stage workload).  Tiles that
+    // stick out of the image have their outside pixels switched off.
+    constexpr int TW = PPW / 2;
     const int ty = t_in / g.tiles_x, tx = t_in - ty * g.tiles_x;
-    const int py = t.p >= g.tile_cols ? 1 : 0;
-    t.pin = (ty * 2 + py) * (int)a.W + tx * g.tile_cols + (t.p - py * g.tile_cols);
+    const int py = t.p >= TW ? 1 : 0;
+    const int y = ty * 2 + py, x = tx * TW + (t.p - py * TW);
+    t.pix_ok = y < (int)a.H && x < (int)a.W;
+    t.pin = y * (int)a.W + x;
   }
-  t.pix_ok = t.pin < g.hw;
   if (!t.pix_ok) t.pin = g.hw - 1;  // clamp: loads stay in range, stores are predicated
   t.pix = (int64_t)t.b * g.hw + t.pin;
   t.h = t.pin / (int)a.W;
@@ -1075,9 +1078,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void
 template <int VEC, int LPP>
 struct Window {
   static constexpr int PPW = 64 / LPP;
-  static constexpr int ROWS = 4;
-  static constexpr int COLS = 2 * PPW > 16 ? 2 * PPW : 16;
+  // twice the tile's width (two rows of PPW/2 pixels) by eight rows: room for the samples'
+  // drift in either direction (against 4 x 2*PPW: 357 -> 338 us on the MVSNet-stage workload)
+  static constexpr int ROWS = 8;
+  static constexpr int COLS = PPW > 8 ? PPW : 8;
   static constexpr int SLOTS = ROWS * COLS;
+  static_assert(SLOTS % 64 == 0, "window_move lists the slots 64 at a time");
   static constexpr int C = VEC * LPP;
   static constexpr int STRIDE = C;      // one slot = C consecutive words: 16-byte lane accesses
   static constexpr int kNone = 0x3fffffff;
@@ -1192,6 +1198,36 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
   }
   oy = ny;
   ox = nx;
+}
+
+// Writes out everything a window holds, at the end of the workgroup: all LDS reads are issued
+// together (the registers of the main loop are free by then), then all the atomics, so the
+// wave waits for the LDS once instead of once per group of texels.
+template <int VEC, int LPP>
+__device__ __forceinline__ void window_flush_all(int oy, int ox, const float *data, float *gview,
+                                                 int srcW, int lane) {
+  using WN = Window<VEC, LPP>;
+  if (oy == WN::kNone) return;
+  wave_sync();  // the last adds are complete and visible
+  constexpr int C = WN::C;
+  constexpr int NI = WN::SLOTS * C / 64;  // instructions of 64 consecutive floats
+  constexpr int BATCH = NI < 32 ? NI : 32;
+  static_assert(NI % BATCH == 0, "whole batches");
+#pragma unroll 1
+  for (int i0 = 0; i0 < NI; i0 += BATCH) {
+    float v[BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) v[u] = data[(i0 + u) * 64 + lane];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int e = (i0 + u) * 64 + lane;  // float index inside the window
+      const int s = e / C, ch = e - s * C;
+      const int ry = s / WN::COLS, rx = s - ry * WN::COLS;
+      const int y = oy + ((ry - oy) & (WN::ROWS - 1)), x = ox + ((rx - ox) & (WN::COLS - 1));
+      // (a slot that was never added to holds zero: texels outside the image never are)
+      if (v[u] != 0.f) atomic_add(gview + ((int64_t)(y * srcW + x) * C + ch), v[u]);
+    }
+  }
 }
 
 // Adds the four tap images of a finished run into the window (a cell that sticks out of the
@@ -1688,7 +1724,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           }
         }
       }
-      if (scl != 0.f) {
+      // (one view per workgroup: a tap offset implies a non-zero factor, phase 1 reprojects
+      // only voxels that have one; one test instead of two per depth)
+      if (NV == 1 ? rec_off[0] >= 0 : scl != 0.f) {
         float cg[VEC];
         {
           const float *raw = cgr[kVoxelGrad ? 0 : jj % PF];
@@ -1844,8 +1882,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   wave_sync();
 #pragma unroll
   for (int n = 0; n < NV; ++n)
-    window_move<VEC, LPP>(oy[n], ox[n], -(1 << 20), -(1 << 20),
-                          s_data + n * WN::SLOTS * WN::STRIDE, s_list, gview[n], srcW, t.lane);
+    window_flush_all<VEC, LPP>(oy[n], ox[n], s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
+                               t.lane);
 
   // pixel-owned gradients: one store when this workgroup saw every depth, otherwise one
   // atomic add per depth segment into the zero-filled outputs
@@ -1894,13 +1932,12 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   constexpr int PPW = 64 / LPP;
   Geometry g;
   g.hw = (int)(H * W);
-  g.tiles_per_image = (g.hw + PPW - 1) / PPW;
-  // two-row tiles where they tile the image exactly
-  g.tile_cols = PPW;
-  g.tiles_x = 1;
-  if (PPW >= 2 && H % 2 == 0 && W % (PPW / 2) == 0) {
-    g.tile_cols = PPW / 2;
-    g.tiles_x = (int)(W / (PPW / 2));
+  if (PPW == 1) {
+    g.tiles_x = (int)W;
+    g.tiles_per_image = g.hw;
+  } else {
+    g.tiles_x = (int)((W + PPW / 2 - 1) / (PPW / 2));
+    g.tiles_per_image = g.tiles_x * (int)((H + 1) / 2);
   }
   const int64_t tiles = B * g.tiles_per_image;
   g.ngroups = ngroups;
