@@ -7,10 +7,11 @@
 // >= C: one lane per channel, so a tap read or a cost-row write of a pixel is one contiguous
 // C-element segment) and one segment of the depth hypotheses, walked in chunks of kDB depths
 // with the views as the middle loop:
-//   phase 1  the first kDB lanes of a pixel reproject the chunk's depths into the view (the
-//            bit-exact code of warp.h) and leave one record per (pixel, depth) in LDS;
-//   phase 2  every lane walks the chunk's depths for its channel; the four taps stay in
-//            registers while consecutive depths fall into the same texel cell.
+//   phase 1  the lanes of a pixel reproject the chunk's depths into a group of views (lane
+//            -> (view of the group, depth): a pixel of 32 lanes serves four views at once; the
+//            bit-exact code of warp.h) and leave one record per (view, pixel, depth) in LDS;
+//   phase 2  view by view, every lane walks the chunk's depths for its channel; the four taps
+//            stay in registers while consecutive depths fall into the same texel cell.
 // Forward: the arithmetic is the reference's literal operand order, every operation rounded
 // separately (cost_volume_kernels_gpu.cu.cc:33-228, cost_volume_kernels_gpu_v2.cu.cc:33-235),
 // views and channels summed in the reference's order, so float and double results are
@@ -18,8 +19,9 @@
 // Backward (:342-577, v2 :349-601): ref_grad and the base-plane gradient are pixel-owned and
 // stay in registers; the source-gradient contributions of a run of depths that share a cell
 // are merged in registers and leave as one atomic add per tap and channel when the cell
-// changes (the reference issues one per voxel); the per-voxel depth gradient is summed over
-// the pixel's lanes in registers and stored once.
+// changes (the reference issues one per voxel) -- a run that is still open at the end of a
+// chunk waits in LDS for the view's turn in the next chunk; the per-voxel depth gradient is
+// summed over the pixel's lanes in registers and stored once.
 #include <type_traits>
 
 #include "internal.h"
@@ -28,11 +30,13 @@ namespace chop {
 
 namespace {
 
-constexpr int kDB = 8;  // depths per chunk
+constexpr int kDB = 8;  // depths per chunk (16 measured slower everywhere: registers)
 
 struct StripGeom {
   int lpp_shift;        // log2(LPP)
   int nseg, seg;        // depth segments, depths per segment (a multiple of kDB)
+  int vg;               // views reprojected together: min(N, max(1, LPP / kDB))
+  int carry;            // backward: open runs survive the end of a chunk (in LDS)
   int64_t tiles;        // ceil(B*H*W / PPW)
 };
 
@@ -74,27 +78,29 @@ __device__ __forceinline__ StripPixel<typename Storage<S>::Real> strip_pixel(con
   return px;
 }
 
-// LDS of one wavefront: kDB records per pixel; a record is addressed [field][pixel*kDB + j].
+// LDS of one wavefront: kDB records per (view of the group, pixel); a record is addressed
+// [field][(view*PPW + pixel)*kDB + j].
 template <typename R>
 struct StripRecords {
-  R *f;      // NF fields of 64/LPP*kDB values each
+  R *f;      // NF fields of vg*PPW*kDB values each
   int *off;  // tap offset inside the view, -1: nothing to do
   int stride;
   __device__ __forceinline__ R &at(int field, int idx) { return f[field * stride + idx]; }
 };
 
 template <typename R, int NF>
-__device__ __forceinline__ StripRecords<R> strip_records(unsigned char *smem, int ppw) {
+__device__ __forceinline__ StripRecords<R> strip_records(unsigned char *smem, int records) {
   StripRecords<R> r;
-  r.stride = ppw * kDB;
+  r.stride = records;
   r.f = reinterpret_cast<R *>(smem);
   r.off = reinterpret_cast<int *>(smem + (size_t)NF * r.stride * sizeof(R));
   return r;
 }
 
+// `records` = vg * PPW * (depths per chunk), then 64 values of staging
 template <typename R>
-constexpr size_t strip_lds_bytes(int nf, int ppw) {
-  return (size_t)ppw * kDB * (nf * sizeof(R) + sizeof(int)) + 64 * sizeof(R);
+constexpr size_t strip_lds_bytes(int nf, int records) {
+  return (size_t)records * (nf * sizeof(R) + sizeof(int)) + 64 * sizeof(R);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -119,9 +125,8 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
   const bool fill = a.default_cost != nullptr;  // the cost-map layers' default for empty voxels
   const R dflt = fill ? *a.default_cost : R(0);
   const int64_t row_step = (int64_t)srcW * C;
-  StripRecords<R> rec = strip_records<R, 4>(smem, ppw);
-  R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw)) - 64;  // CORR: products of a pixel
-  const int ridx = p * kDB;
+  StripRecords<R> rec = strip_records<R, 4>(smem, ppw * g.vg * kDB);
+  R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw * g.vg * kDB)) - 64;  // CORR: products of a pixel
 
   for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
     R acc[kDB];
@@ -132,27 +137,34 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
       arg[jj] = -1;
       kcnt[jj] = 0;
     }
-    for (int n = 0; n < N; ++n) {
-      const int64_t cam = (int64_t)px.b * N + n;
-      strip_sync();  // the records of the view before have been read
-      for (int j = cl; j < kDB; j += lpp) {
-        const int d = d0 + j;
-        int off = -1;
-        Sample<R> s;
-        s.k00 = s.k01 = s.k11 = s.k10 = R(0);
-        if (d < d_hi) {
-          const R depth = a.depth_grid ? a.depth_grid[px.pix * D + d]
-                                       : base + a.offsets[(int64_t)px.b * D + d];
-          project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
-          if (s.state == 2) off = (s.fh * srcW + s.fw) * C;
-        }
-        rec.off[ridx + j] = off;
-        rec.at(0, ridx + j) = s.k00;
-        rec.at(1, ridx + j) = s.k01;
-        rec.at(2, ridx + j) = s.k11;
-        rec.at(3, ridx + j) = s.k10;
+    for (int n0 = 0; n0 < N; n0 += g.vg) {
+    const int nv = min(g.vg, N - n0);
+    strip_sync();  // the records of the views before have been read
+    for (int item = cl; item < nv * kDB; item += lpp) {
+      const int nl = item / kDB, j = item - nl * kDB;
+      const int64_t cam = (int64_t)px.b * N + n0 + nl;
+      const int d = d0 + j;
+      int off = -1;
+      Sample<R> s;
+      s.k00 = s.k01 = s.k11 = s.k10 = R(0);
+      if (d < d_hi) {
+        const R depth = a.depth_grid ? a.depth_grid[px.pix * D + d]
+                                     : base + a.offsets[(int64_t)px.b * D + d];
+        project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
+        if (s.state == 2) off = (s.fh * srcW + s.fw) * C;
       }
-      strip_sync();
+      const int r = (nl * ppw + p) * kDB + j;
+      rec.off[r] = off;
+      rec.at(0, r) = s.k00;
+      rec.at(1, r) = s.k01;
+      rec.at(2, r) = s.k11;
+      rec.at(3, r) = s.k10;
+    }
+    strip_sync();
+    for (int nl = 0; nl < nv; ++nl) {
+      const int n = n0 + nl;
+      const int ridx = (nl * ppw + p) * kDB;
+      const int64_t cam = (int64_t)px.b * N + n;
       const S *view = a.src + cam * srcH * srcW * C + (ch_ok ? cl : 0);
       int cur = -1;
       R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
@@ -190,13 +202,20 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
         ++kcnt[jj];
       }
     }
+    }  // group of views
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) {
       const int d = d0 + jj;
       if (d >= d_hi) break;
       const int64_t i = px.pix * D + d;
       if (REDUCE == 0) {
-        if (kcnt[jj] > 0) acc[jj] = acc[jj] / static_cast<R>(kcnt[jj]);
+        // the mean: halving and quartering are exact, so only other counts pay for a division
+        if (kcnt[jj] == 2)
+          acc[jj] = acc[jj] * R(0.5);
+        else if (kcnt[jj] == 4)
+          acc[jj] = acc[jj] * R(0.25);
+        else if (kcnt[jj] > 2)
+          acc[jj] = acc[jj] / static_cast<R>(kcnt[jj]);
         if (px.ok && cl == 0) a.mask[i] = kcnt[jj];
       } else if (out_ok) {
         a.mask[i * OC + cl] = arg[jj];
@@ -232,19 +251,29 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
   const bool per_voxel = a.depth_grid != nullptr, want_depth = a.depth_grad != nullptr;
   const int64_t row_step = (int64_t)srcW * C;
-  // fields: the four weights, dh, dw, the two depth-chain factors, the view count as a real
-  StripRecords<R> rec = strip_records<R, 9>(smem, ppw);
-  const int ridx = p * kDB;
+  // fields: the four weights, dh, dw, the two depth-chain factors, 1 / view count
+  StripRecords<R> rec = strip_records<R, 9>(smem, ppw * g.vg * kDB);
+  // open runs between two chunks: per view the cell and its four tap sums, one slot per lane
+  // (a lane only ever reads its own slots back)
+  R *s_run = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(9, ppw * g.vg * kDB));
+  int *s_cur = reinterpret_cast<int *>(s_run + (size_t)N * 4 * 64);
+  const bool carry = g.carry != 0;
+  if (carry)
+    for (int n = 0; n < N; ++n) s_cur[n * 64 + lane] = -1;
   R racc = R(0), dpart = R(0);
 
   for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
     R dvox[kDB];
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) dvox[jj] = R(0);
-    for (int n = 0; n < N; ++n) {
-      const int64_t cam = (int64_t)px.b * N + n;
-      strip_sync();
-      for (int j = cl; j < kDB; j += lpp) {
+    for (int n0 = 0; n0 < N; n0 += g.vg) {
+    const int nv = min(g.vg, N - n0);
+    strip_sync();
+    for (int item = cl; item < nv * kDB; item += lpp) {
+      {
+        const int nl = item / kDB, j = item - nl * kDB;
+        const int64_t cam = (int64_t)px.b * N + n0 + nl;
+        const int ridx = (nl * ppw + p) * kDB;
         const int d = d0 + j;
         int off = -1;
         Sample<R> s;
@@ -262,7 +291,7 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
               const R zz = s.z * s.z;
               fh = (s.h_coef * s.z - s.z_coef * s.h3d) / zz;
               fw = (s.w_coef * s.z - s.z_coef * s.w3d) / zz;
-              cnt = static_cast<R>(m0);
+              cnt = R(1) / static_cast<R>(m0);
             }
           }
         }
@@ -277,13 +306,22 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         rec.at(7, ridx + j) = fw;
         rec.at(8, ridx + j) = cnt;
       }
-      strip_sync();
-      const int64_t view_off = cam * srcH * srcW * C + (ch_ok ? cl : 0);
+    }
+    strip_sync();
+    for (int nl = 0; nl < nv; ++nl) {
+      const int n = n0 + nl;
+      const int ridx = (nl * ppw + p) * kDB;
+      const int64_t view_off = ((int64_t)px.b * N + n) * srcH * srcW * C + (ch_ok ? cl : 0);
       const S *view = a.src + view_off;
       Acc *gview = src_grad + view_off;
-      int cur = -1;
+      int cur = -1, have = -1;  // cell of the open run, cell whose taps are in registers
       R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
       R g00 = R(0), g01 = R(0), g11 = R(0), g10 = R(0);
+      if (carry) {
+        cur = s_cur[n * 64 + lane];
+        g00 = s_run[(n * 4 + 0) * 64 + lane], g01 = s_run[(n * 4 + 1) * 64 + lane];
+        g11 = s_run[(n * 4 + 2) * 64 + lane], g10 = s_run[(n * 4 + 3) * 64 + lane];
+      }
       auto flush = [&]() {
         if (cur >= 0 && ch_ok) {
           Acc *q = gview + cur;
@@ -302,6 +340,9 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         if (off != cur) {
           flush();
           cur = off;
+        }
+        if (off != have) {
+          have = off;
           const S *q = view + off;
           v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
           v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
@@ -312,14 +353,16 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
                 k10 = rec.at(3, ridx + jj);
         const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
         const R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
-        const R cnt = rec.at(8, ridx + jj);
+        // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
+        // reference's division (one division per voxel in phase 1 instead of one per element)
+        const R inv = rec.at(8, ridx + jj);
         R gv;
         if (CORR == 0) {
           const R diff = smp - ref_c;
-          gv = REDUCE == 0 ? R(2) * diff * cg / cnt : R(2) * diff * cg;  // :439, :560
+          gv = REDUCE == 0 ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
           racc += -gv;
         } else {
-          gv = REDUCE == 0 ? cg / cnt : cg;  // v2 :461, :583
+          gv = REDUCE == 0 ? cg * inv : cg;  // v2 :461, :583
           racc += gv * smp;
           gv = gv * ref_c;
         }
@@ -338,8 +381,15 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
             dpart += dl;
         }
       }
-      flush();
+      if (carry) {
+        s_cur[n * 64 + lane] = cur;
+        s_run[(n * 4 + 0) * 64 + lane] = g00, s_run[(n * 4 + 1) * 64 + lane] = g01;
+        s_run[(n * 4 + 2) * 64 + lane] = g11, s_run[(n * 4 + 3) * 64 + lane] = g10;
+      } else {
+        flush();
+      }
     }
+    }  // group of views
     if (per_voxel && want_depth) {
 #pragma unroll
       for (int jj = 0; jj < kDB; ++jj) {
@@ -348,6 +398,20 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         // every voxel is stored, zeros on the ones the mask skips (v2 :375-378, :477)
         if (d < d_hi && px.ok && cl == 0) a.depth_grad[px.pix * D + d] = tot;
       }
+    }
+  }
+  if (carry && ch_ok) {
+    // the runs still open after the last chunk
+    for (int n = 0; n < N; ++n) {
+      const int cur = s_cur[n * 64 + lane];
+      if (cur < 0) continue;
+      Acc *q = src_grad + ((int64_t)px.b * N + n) * srcH * srcW * C + cl + cur;
+      const R g00 = s_run[(n * 4 + 0) * 64 + lane], g01 = s_run[(n * 4 + 1) * 64 + lane];
+      const R g11 = s_run[(n * 4 + 2) * 64 + lane], g10 = s_run[(n * 4 + 3) * 64 + lane];
+      if (g00 != R(0)) atomic_add(q, (Acc)g00);
+      if (g01 != R(0)) atomic_add(q + C, (Acc)g01);
+      if (g11 != R(0)) atomic_add(q + C + row_step, (Acc)g11);
+      if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
     }
   }
   if (ch_ok) {
@@ -369,18 +433,27 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
 }
 
 template <typename S>
+constexpr size_t strip_run_bytes(int64_t N) {
+  return (size_t)N * 64 * (4 * sizeof(typename Storage<S>::Real) + sizeof(int));
+}
+
+template <typename S>
 StripGeom strip_geometry(const Args<S> &a) {
   StripGeom g;
   g.lpp_shift = 0;
   while ((1 << g.lpp_shift) < a.C) ++g.lpp_shift;
   const int ppw = 64 >> g.lpp_shift;
   g.tiles = (a.pixels() + ppw - 1) / ppw;
+  const int lpp = 1 << g.lpp_shift;
+  g.vg = lpp / kDB < 1 ? 1 : (int)(lpp / kDB < a.N ? lpp / kDB : a.N);
   // enough wavefronts to fill 256 compute units several times over, segments of whole chunks
   int nseg = 1;
-  while (nseg < 16 && g.tiles * nseg < 256 * 16 && a.D / (nseg * 2) >= kDB) nseg *= 2;
+  while (nseg < 16 && g.tiles * nseg < 256 * 80 && a.D / (nseg * 2) >= 2 * kDB) nseg *= 2;
   const int per = (int)((a.D + nseg - 1) / nseg);
   g.seg = (per + kDB - 1) / kDB * kDB;
   g.nseg = (int)((a.D + g.seg - 1) / g.seg);
+  // carried runs: N * 64 lanes * (4 sums + cell); given up beyond 16 KiB
+  g.carry = strip_run_bytes<S>(a.N) <= 16384;
   return g;
 }
 
@@ -401,7 +474,7 @@ template <typename S>
 hipError_t launch_strip_forward(const Args<S> &a, hipStream_t stream) {
   using R = typename Storage<S>::Real;
   const StripGeom g = strip_geometry(a);
-  const size_t smem = strip_lds_bytes<R>(4, 64 >> g.lpp_shift);
+  const size_t smem = strip_lds_bytes<R>(4, (64 >> g.lpp_shift) * g.vg * kDB);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
   if (a.corr == SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
@@ -436,7 +509,8 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
         (err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(R), stream)) != hipSuccess)
       return err;
   }
-  const size_t smem = strip_lds_bytes<R>(9, 64 >> g.lpp_shift);
+  const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB) +
+                      (g.carry ? strip_run_bytes<S>(a.N) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
   if (a.corr == SQUARED_DIFFERENCE) {
     if (a.reduce == 0)

@@ -1531,9 +1531,12 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     float4 r_wts[NV], r_dwt[NV];
     bool chunk_out[NV];  // some cell of this chunk (or the open one) sticks out of the window
     // Issue the loads of this chunk's cost_grad rows now, unconditionally, so that the
-    // reprojection below overlaps their latency.  Streaming loads: cached ones let the
-    // next view's workgroup hit L2 more often (690 -> 660 MB fetched) and save 10 us here,
-    // but leave the caches full of these rows and cost the next forward launch 25 us.
+    // reprojection below overlaps their latency.  Streaming loads, although the workgroups of
+    // a tile's views read the same rows and only about half of the later reads find them in
+    // L2.  Cached loads for every view but the last fetch 676 instead of 830 MB on the
+    // two-view benchmark tensors and save 2 % with warm caches, but the rows they leave
+    // behind in L2 and the memory-side cache cost the next forward launch 5 us, and after
+    // other work has filled the caches with dirty lines they are 3 % slower than streaming.
     float cgr[kVoxelGrad ? 1 : PF][VEC];
     int mrow[kMaskRows ? PF : 1][VEC];
     auto load_rows = [&](int first) {
@@ -1942,8 +1945,8 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   const int64_t tiles = B * g.tiles_per_image;
   g.ngroups = ngroups;
   g.vper = vper;
-  // the backward kernel (the one with view groups) runs more, lighter waves per CU
-  g.nseg = choose_segments(tiles * ngroups, D, LPP, vper > 0 ? 256 * 4 * 20 : 256 * 4 * 10);
+  // twenty waves per SIMD over the launch: the tail of a launch with fewer is measurable
+  g.nseg = choose_segments(tiles * ngroups, D, LPP, 256 * 4 * 20);
   const int per_seg = (int)((D + g.nseg - 1) / g.nseg);
   g.seg = ((per_seg + LPP - 1) / LPP) * LPP;
   g.nseg = (int)((D + g.seg - 1) / g.seg);
