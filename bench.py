@@ -36,10 +36,13 @@ class Runner:
     def __init__(self, wl, torch, lib):
         self.wl, self.torch, self.lib = wl, torch, lib
         t = wl.tensors
-        td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[wl.storage]
-        self.storage_code = {"f32": 0, "f16": 1, "bf16": 2}[wl.storage]
+        td = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16,
+              "f64": torch.float64}[wl.storage]
+        self.storage_code = {"f32": 0, "f16": 1, "bf16": 2, "f64": 0}[wl.storage]
+        self.f64 = wl.storage == "f64"  # depths, cameras and depth gradients are float64 too
+        real = torch.float64 if self.f64 else None
         d = "cuda:0"
-        up = lambda k, dt=None: (torch.from_numpy(t[k]).to(d) if dt is None
+        up = lambda k, dt=real: (torch.from_numpy(t[k]).to(d) if dt is None
                                  else torch.from_numpy(t[k]).to(d).to(dt))
         self.ref, self.src = up("ref", td), up("src", td)
         self.Rs, self.Ts = up("Rs"), up("Ts")
@@ -62,7 +65,7 @@ class Runner:
         self.ref_grad = torch.empty_like(self.ref)
         self.src_grad = torch.empty_like(self.src)
         self.depth_grad = torch.empty((B, H, W, D) if self.v2 else (B, H, W, 1),
-                                      dtype=torch.float32, device=d)
+                                      dtype=real or torch.float32, device=d)
         self.dims = (B, H, W, wl.C, D, wl.N, H, W)
         self.ws = None
         self.ws_bytes = 0
@@ -103,9 +106,9 @@ class Runner:
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
                                              p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
         else:
-            rc = lib.chop_cost_volume_fwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
-                                              p(self.base_plane), p(self.offsets), p(self.Rs),
-                                              p(self.Ts), p(self.cost), p(self.mask))
+            fn = lib.chop_cost_volume_fwd_f64 if self.f64 else lib.chop_cost_volume_fwd_f32
+            rc = fn(s, self.red, 1, *self.dims, p(self.ref), p(self.src), p(self.base_plane),
+                    p(self.offsets), p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
         if rc:
             raise RuntimeError(lib.chop_last_error_string().decode())
 
@@ -143,9 +146,9 @@ class Runner:
                                              p(self.Rs), p(self.Ts), *tail, p(self.ws),
                                              self.ws_bytes)
         else:
-            rc = lib.chop_cost_volume_bwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
-                                              p(self.base_plane), p(self.offsets), p(self.Rs),
-                                              p(self.Ts), *tail)
+            fn = lib.chop_cost_volume_bwd_f64 if self.f64 else lib.chop_cost_volume_bwd_f32
+            rc = fn(s, self.red, 1, *self.dims, p(self.ref), p(self.src), p(self.base_plane),
+                    p(self.offsets), p(self.Rs), p(self.Ts), *tail)
         if rc:
             raise RuntimeError(lib.chop_last_error_string().decode())
 
@@ -309,6 +312,13 @@ def main():
                     help="time CostVolumeV3 with this many channel groups on the workload's tensors")
     ap.add_argument("--feature", action="store_true",
                     help="time FeatureAggregate on the workload's tensors")
+    ap.add_argument("--float64", action="store_true",
+                    help="time a float32 CostVolume workload's tensors as float64 (strip kernels)")
+    ap.add_argument("--channels", type=int, default=0, metavar="C",
+                    help="keep only the first C feature channels of a float32 CostVolume workload")
+    ap.add_argument("--kernel-family", choices=["auto", "general", "strip"], default="auto",
+                    help="force the one-thread-per-element or the strip kernels instead of the "
+                         "library's own choice")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
@@ -320,8 +330,21 @@ def main():
     from custom_helper_op_amd import _lib
     from custom_helper_op_amd.configs import make_workload
     lib = _lib.load()
+    lib.chop_set_kernel_family({"auto": 0, "general": 1, "strip": 2}[a.kernel_family])
     wl = make_workload(a.workload, with_cost_grad=False)
     wl.reduce_method = a.reduce
+    if a.float64 or a.channels:
+        if wl.op != "v1" or wl.storage != "f32" or a.aggregate or a.v3 or a.feature:
+            sys.exit("bench.py: --float64 / --channels need a float32 CostVolume workload (1, 2 or 5)")
+        if a.channels:
+            if not 1 <= a.channels <= wl.C:
+                sys.exit("bench.py: --channels must be 1..%d for this workload" % wl.C)
+            import numpy as np
+            wl.C = a.channels
+            for k in ("ref", "src"):
+                wl.tensors[k] = np.ascontiguousarray(wl.tensors[k][..., :wl.C])
+        if a.float64:
+            wl.storage = "f64"
     if a.aggregate:
         if wl.op != "v1" or wl.storage != "f32":
             sys.exit("bench.py: --aggregate needs a float32 CostVolume workload (1, 2 or 5)")
@@ -332,6 +355,11 @@ def main():
         wl.op = "v3" if a.v3 else "feat"
         wl.groups = a.v3 if a.v3 else 1
     r = Runner(wl, torch, lib)
+    r.forward()
+    served = [lib.chop_last_kernel_family()]
+    r.backward()
+    served.append(lib.chop_last_kernel_family())
+    served = "/".join({1: "general", 2: "tiled", 3: "strip"}.get(c, str(c)) for c in served)
     for _ in range(a.warmup):
         r.forward()
         r.backward()
@@ -366,7 +394,8 @@ def main():
     traffic_source = None
     try:  # HBM bytes per launch from rocprofv3 counters of a separate run of this command
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            t = json.load(f)[wl.name if wl.op in ("v1", "v2") and a.reduce == "MEAN" else "-"][dominant]
+            plain = wl.op in ("v1", "v2") and a.reduce == "MEAN" and not (a.float64 or a.channels)
+            t = json.load(f)[wl.name if plain and a.kernel_family == "auto" else "-"][dominant]
         traffic = t["fetch_bytes"] + t["write_bytes"]
         traffic_source = "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE/WRITE_SIZE of a separate run)"
     except (OSError, KeyError, ValueError):
@@ -385,7 +414,8 @@ def main():
                       "feat": "FeatureAggregate"}[wl.op],
             wl.B, wl.N, wl.H, wl.W,
             wl.C, wl.D, " G%d" % wl.groups if wl.op in ("v2", "v3") else "", wl.storage),
-            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True},
+            "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True,
+            "kernels": served},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "timing": "HIP events on the launch stream, caches overwritten before each call, median",
@@ -411,7 +441,7 @@ def main():
             "backward_frac": bwd_b / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "fwd_bwd_frac": out["roofline"]["fwd_bwd_frac"],
             "voxels_per_s": wl.voxels / ((fwd_ms + bwd_ms) * 1e-3)}
-    if not a.no_cpu_baseline:
+    if not a.no_cpu_baseline and not a.float64:  # (the checker is timed in the workload's own type)
         out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
 
