@@ -643,6 +643,49 @@ def test_five_views(oracle, C, reduce):
         assert_forward_close(host(cost), want_cost, atol=1e-5)
 
 
+# ---- strip kernels: several view groups, with and without carried runs --------------------------
+@pytest.mark.parametrize("C,N,dtype", [(5, 9, np.float64), (40, 9, np.float64), (24, 7, np.float32),
+                                       (3, 17, np.float32), (33, 3, np.float64)])
+@pytest.mark.parametrize("reduce", ["MEAN", "MIN"])
+def test_strip_many_views(oracle, C, N, dtype, reduce):
+    """The strip kernels reproject min(N, max(1, lanes per pixel / 8)) views per phase 1 and keep
+    the runs that are open at the end of a chunk in LDS as long as that takes at most 16 KiB
+    (N <= 7 in float64, N <= 14 in float32).  These shapes cover one view at a time (C = 3, 5),
+    groups of four and eight with a remainder (C = 24, 33, 40) and both sides of the limit;
+    D = 21 leaves a ragged last chunk."""
+    B, H, W, D = 1, 10, 14, 21
+    t = reference_test_case(3, B, N, H, W, C, D, dtype, seed=C + N)
+    t["Ts"] = (t["Ts"] + np.linspace(-1, 1, N)[None, :, None]).astype(dtype)   # N different views
+    args = tuple(t[k] for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts"))
+    want_cost, want_mask = oracle.cost_volume_fwd(*args, reduce)
+    _lib.load().chop_set_kernel_family(2)
+    cost, mask = chop.cost_volume_raw(*_v1_inputs(t), reduce)
+    _assert_family(2)
+    assert np.array_equal(host(mask), want_mask)
+    assert np.array_equal(host(cost), want_cost)   # literal operand order: bit-identical
+    cg = np.random.default_rng(C).standard_normal(want_cost.shape).astype(dtype)
+    want = oracle.cost_volume_bwd(*args, cg, want_mask, reduce)
+    got = chop.cost_volume_grad(*_v1_inputs(t), dev(cg), mask, reduce)
+    _assert_family(2)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+    if C in (24, 40):
+        groups = 8
+        depth_grid = (t["base_plane"] + t["offsets"][:, None, None, :]).astype(dtype)
+        a2 = (t["ref"], t["src"], depth_grid, t["Rs"], t["Ts"])
+        want_cost, want_mask = oracle.cost_volume_v2_fwd(*a2, reduce, groups)
+        cost, mask = chop.cost_volume_v2_raw(*[dev(x) for x in a2], reduce, groups)
+        _assert_family(2)
+        assert np.array_equal(host(mask), want_mask)
+        assert np.array_equal(host(cost), want_cost)
+        cg = np.random.default_rng(N).standard_normal(want_cost.shape).astype(dtype)
+        want = oracle.cost_volume_v2_bwd(*a2, cg, want_mask, reduce, groups)
+        got = chop.cost_volume_grad_v2(*[dev(x) for x in a2], dev(cg), mask, reduce, groups)
+        _assert_family(2)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+
+
 # ---- samples that jump far between consecutive depths ------------------------------------------
 @pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
 def test_backward_cells_outside_the_scatter_window(oracle, C):
