@@ -47,10 +47,11 @@ class Runner:
         self.ref, self.src = up("ref", td), up("src", td)
         self.Rs, self.Ts = up("Rs"), up("Ts")
         self.v2 = wl.op == "v2"
+        self.grid = wl.op == "v1" and wl.grid_form  # squared difference over a depth grid (16-bit only)
         self.agg = wl.op == "agg"
         self.v3, self.feat = wl.op == "v3", wl.op == "feat"
         self.red = 0 if wl.reduce_method == "MEAN" else 1
-        if self.v2:
+        if self.v2 or self.grid:
             self.depth_grid = up("depth_grid")
         else:
             self.base_plane, self.offsets = up("base_plane"), up("offsets")
@@ -64,7 +65,7 @@ class Runner:
                                      generator=gen).to(td)
         self.ref_grad = torch.empty_like(self.ref)
         self.src_grad = torch.empty_like(self.src)
-        self.depth_grad = torch.empty((B, H, W, D) if self.v2 else (B, H, W, 1),
+        self.depth_grad = torch.empty((B, H, W, D) if self.v2 or self.grid else (B, H, W, 1),
                                       dtype=real or torch.float32, device=d)
         self.dims = (B, H, W, wl.C, D, wl.N, H, W)
         self.ws = None
@@ -101,6 +102,10 @@ class Runner:
             rc = lib.chop_feature_aggregate_fwd_f32(s, 1, *self.dims, p(self.src),
                                                     p(self.base_plane), p(self.offsets), p(self.Rs),
                                                     p(self.Ts), p(self.cost), p(self.mask))
+        elif self.grid:
+            rc = lib.chop_cost_volume_fwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
+                                             p(self.src), None, None, p(self.depth_grid),
+                                             p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
         elif self.storage_code:
             rc = lib.chop_cost_volume_fwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
@@ -140,6 +145,11 @@ class Runner:
                                                     p(self.base_plane), p(self.offsets), p(self.Rs),
                                                     p(self.Ts), p(self.cost_grad), p(self.mask),
                                                     p(self.src_grad), p(self.depth_grad))
+        elif self.grid:
+            rc = lib.chop_cost_volume_bwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
+                                             p(self.src), None, None, p(self.depth_grid),
+                                             p(self.Rs), p(self.Ts), *tail, p(self.ws),
+                                             self.ws_bytes)
         elif self.storage_code:
             rc = lib.chop_cost_volume_bwd_16(s, self.storage_code, self.red, 1, *self.dims, p(self.ref),
                                              p(self.src), p(self.base_plane), p(self.offsets), None,
@@ -271,10 +281,13 @@ def other_configs(torch, lib, make_workload, skip_index, scratch):
     """Forward / backward event times of the BASELINE configurations the headline line is not
     quoted on, each against its own algorithmic bytes (cold-cache, median of 5)."""
     out = {}
-    for index in (1, 2, 3, 4, 5):
+    for index, grid_form in ((1, False), (2, False), (3, False), (3, True), (4, False), (5, False)):
         if index == skip_index:
             continue
         wl = make_workload(index, with_cost_grad=False)
+        if grid_form:  # the cascade stage's exact per-pixel hypotheses, coarse * (1 + 0.02 k)
+            wl.grid_form = True
+            wl.name += "_depth_grid"
         r = Runner(wl, torch, lib)
         for _ in range(2):
             r.forward()
@@ -284,9 +297,9 @@ def other_configs(torch, lib, make_workload, skip_index, scratch):
         fwd_b, bwd_b = wl.algorithmic_bytes()
         frac = lambda b, ms: b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         out[wl.name] = {
-            "workload": "%s B%d N%d %dx%d C%d D%d %s" % (
+            "workload": "%s B%d N%d %dx%d C%d D%d %s%s" % (
                 {"v1": "CostVolume", "v2": "CostVolumeV2"}[wl.op], wl.B, wl.N, wl.H, wl.W, wl.C,
-                wl.D, wl.storage),
+                wl.D, wl.storage, " over depth_grid" if grid_form else ""),
             "voxels": wl.voxels, "forward_ms": fwd_ms, "backward_ms": bwd_ms,
             "forward_frac": frac(fwd_b, fwd_ms), "backward_frac": frac(bwd_b, bwd_ms),
             "fwd_bwd_frac": frac(fwd_b + bwd_b, fwd_ms + bwd_ms),

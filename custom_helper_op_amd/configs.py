@@ -36,6 +36,7 @@ class Workload:
     backward: bool = True
     reduce_method: str = "MEAN"
     half_centor: bool = True
+    grid_form: bool = False  # "v1" with per-voxel hypotheses (depth_grid) instead of plane + offsets
     seed: int = 0
     tensors: Dict[str, np.ndarray] = field(default_factory=dict)
 
@@ -64,7 +65,7 @@ class Workload:
         ref = px * self.C * e
         src = self.B * self.N * self.H * self.W * self.C * e
         cams = self.B * self.N * 12 * f
-        if self.op != "v2":
+        if self.op != "v2" and not self.grid_form:
             depth_in = px * f + self.B * self.D * f
             depth_grad = px * f
         else:
