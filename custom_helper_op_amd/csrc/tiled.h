@@ -495,10 +495,24 @@ constexpr int forward_squares_words(int lpp) { return lpp > 1 ? 64 * (4 * lpp + 
 // the squared difference / per-group maximum of the correlation with the winning view as
 // mask (-1: none).  The winner must be the reference's, so that reduce uses the literal
 // operand order with every operation rounded separately instead of the fused chains.
+// Minimum waves per SIMD the register allocator has to leave room for (mean of the squared
+// difference or of the group correlation only: the MIN / MAX reduces keep winner indices per
+// depth and channel and would spill).  Five and six views: left alone the compiler takes ~140
+// registers (three waves); held to 128 it needs no scratch, and the fourth wave hides the tap
+// gathers of wide-baseline views (stress workload forward 5.17 -> 4.45 ms).  Three and four
+// views at four lanes per pixel: 102 -> 87 registers without scratch, five waves instead of
+// four (f16 cascade workload forward 122 -> 113 us cold); the other widths would spill.
+constexpr int forward_min_waves(int lpp, int nv, int corr, int reduce) {
+  if (corr > 1 || reduce != 0) return 1;
+  return nv >= 5 ? 4 : (nv >= 3 && lpp == 4) ? 5 : 1;
+}
+
 template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0>
 // At most five waves per SIMD: with six (the two-view instantiation needs only 80 VGPRs)
-// the waves of a CU evict each other's taps from L1 and the kernel is 6 % slower.
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(1, 5))) void forward_kernel(
+// the waves of a CU evict each other's taps from L1 and the kernel is 6 % slower.  The lower
+// bound: see forward_min_waves.
+__global__ __launch_bounds__(64)
+__attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))) void forward_kernel(
     const Args<S> a, const Geometry g) {
   constexpr int PPW = 64 / LPP;
   extern __shared__ __align__(16) unsigned char smem[];
