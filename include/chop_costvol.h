@@ -317,6 +317,10 @@ int chop_cost_volume_v2_fwd_fill_f64(void *stream, int reduce, int half_centor, 
  * `depth_grid` non-NULL selects per-pixel hypotheses for the V1 squared-difference
  * reduce (base_plane/offsets are then ignored and the third gradient has the shape of
  * depth_grid).
+ * With CHOP_REDUCE_MIN an element no view reached keeps the fp32 seed rounded to the storage
+ * type: the largest float becomes +infinity in both 16-bit types, the group correlation's
+ * smallest normal float stays what it is in bfloat16 and becomes 0 in half; the mask entry
+ * (-1) marks such an element, as in the float ops.
  * The backward accumulates source/reference gradients in fp32 inside `workspace`
  * (device memory, 256-byte aligned, at least chop_cost_volume_bwd16_workspace_bytes). */
 size_t chop_cost_volume_bwd16_workspace_bytes(int64_t B, int64_t H, int64_t W, int64_t C,

@@ -135,3 +135,69 @@ def test_random_shape_other_ops(oracle, seed):
     got_g = chop.feature_aggregate_grad(*df, dev(g), mask, half)
     for a, b in zip(got_g, want_g):
         assert_backward_close(host(a), b, tol)
+
+
+@pytest.mark.parametrize("seed", range(200, 224))
+def test_random_shape_16bit_storage(oracle, seed):
+    """float16 / bfloat16 feature storage with float32 arithmetic: the float32 oracle on the
+    quantised inputs, masks bit-exact, values within 1e-2 (the outputs themselves are rounded to
+    11 or 8 significant bits).  CostVolume over planes and over a depth grid, CostVolumeV2."""
+    import torch
+    from custom_helper_op_amd.configs import quantise
+    from gpu_util import TORCH_DTYPE, rms
+    t, shape, _, reduce, half, groups = _case(seed)
+    B, N, H, W, C, D = shape
+    storage = "f16" if seed % 2 else "bf16"
+    print("\n[case] seed %d: B%d N%d %dx%d C%d D%d %s %s half=%s groups=%d" % (
+        seed, B, N, H, W, C, D, storage, reduce, half, groups), flush=True)
+    td = TORCH_DTYPE[storage]
+    f32 = np.float32
+    ref, src = quantise(t["ref"].astype(f32), storage), quantise(t["src"].astype(f32), storage)
+    bp, off, Rs, Ts = (t[k].astype(f32) for k in ("base_plane", "offsets", "Rs", "Ts"))
+    rng = np.random.default_rng(seed)
+
+    def close(got, want, mask=None):
+        if mask is not None and reduce == "MIN":
+            # an element no view reached keeps the float seed, rounded to the storage type:
+            # FLT_MAX becomes +inf in both 16-bit types, the correlation's 1.18e-38 stays (bf16)
+            # or becomes 0 (f16); the mask (-1) is what marks such an element
+            empty = mask < 0
+            assert np.all(np.isinf(got[empty]) | (np.abs(got[empty]) < 1e-37))
+            got, want = got[~empty], want[~empty]
+        np.testing.assert_allclose(got, want, rtol=1e-2, atol=1e-2 * max(rms(want), 1e-30))
+
+    want_cost, want_mask = oracle.cost_volume_fwd(ref, src, bp, off, Rs, Ts, reduce, half)
+    ins = [dev(ref, td), dev(src, td), dev(bp), dev(off), dev(Rs), dev(Ts)]
+    cost, mask = chop.cost_volume_raw(*ins, reduce, half)
+    assert cost.dtype == td
+    assert np.array_equal(host(mask), want_mask)
+    close(host(cost), want_cost, want_mask)
+    cg = quantise(rng.standard_normal(want_cost.shape).astype(f32), storage)
+    want = oracle.cost_volume_bwd(ref, src, bp, off, Rs, Ts, cg, want_mask, reduce, half)
+    got = chop.cost_volume_grad(*ins, dev(cg, td), mask, reduce, half)
+    assert got[2].dtype == torch.float32
+    for g, w in zip(got, want):
+        close(host(g), w)
+
+    grid = (bp * (1.0 + 0.01 * (np.arange(D, dtype=f32) - D // 2))[None, None, None]).astype(f32)
+    want_cost, want_mask = oracle.cost_volume_grid_fwd(ref, src, grid, Rs, Ts, reduce, half)
+    gins = [dev(ref, td), dev(src, td), None, None, dev(Rs), dev(Ts)]
+    cost, mask = chop.cost_volume_raw(*gins, reduce, half, depth_grid=dev(grid))
+    assert np.array_equal(host(mask), want_mask)
+    close(host(cost), want_cost, want_mask)
+    want = oracle.cost_volume_grid_bwd(ref, src, grid, Rs, Ts, cg, want_mask, reduce, half)
+    got = chop.cost_volume_grad(*gins, dev(cg, td), mask, reduce, half, depth_grid=dev(grid))
+    assert got[2].shape == (B, H, W, D)
+    for g, w in zip(got, want):
+        close(host(g), w)
+
+    want_cost, want_mask = oracle.cost_volume_v2_fwd(ref, src, grid, Rs, Ts, reduce, groups, half)
+    vins = [dev(ref, td), dev(src, td), dev(grid), dev(Rs), dev(Ts)]
+    cost, mask = chop.cost_volume_v2_raw(*vins, reduce, groups, half)
+    assert np.array_equal(host(mask), want_mask)
+    close(host(cost), want_cost, want_mask)
+    cg = quantise(rng.standard_normal(want_cost.shape).astype(f32), storage)
+    want = oracle.cost_volume_v2_bwd(ref, src, grid, Rs, Ts, cg, want_mask, reduce, groups, half)
+    got = chop.cost_volume_grad_v2(*vins, dev(cg, td), mask, reduce, groups, half)
+    for g, w in zip(got, want):
+        close(host(g), w)
