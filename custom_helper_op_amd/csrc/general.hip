@@ -189,7 +189,7 @@ __global__ __launch_bounds__(kBlock) void general_backward_kernel(const Args<S> 
   }
 }
 
-__global__ __launch_bounds__(kBlock) void fill_zero_kernel(unsigned char *p, size_t bytes) {
+__device__ __forceinline__ void zero_range(unsigned char *p, size_t bytes) {
   // head up to 16-byte alignment, 16-byte body, byte tail
   const size_t mis = (size_t)(-(intptr_t)p) & 15u;
   const size_t head = mis < bytes ? mis : bytes;
@@ -204,11 +204,30 @@ __global__ __launch_bounds__(kBlock) void fill_zero_kernel(unsigned char *p, siz
   if (tid < bytes - tail_at) p[tail_at + tid] = 0;
 }
 
+__global__ __launch_bounds__(kBlock) void fill_zero_kernel(unsigned char *p, size_t bytes) {
+  zero_range(p, bytes);
+}
+
+__global__ __launch_bounds__(kBlock) void fill_zero_ranges_kernel(const ZeroRanges r) {
+  for (int i = 0; i < r.count; ++i) zero_range(r.ptr[i], r.bytes[i]);
+}
+
 template <typename S>
 __global__ __launch_bounds__(kBlock) void narrow_kernel(const float *from, S *to, int64_t count) {
   for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < count;
        k += (int64_t)gridDim.x * kBlock)
     Storage<S>::store(to + k, from[k]);
+}
+
+template <typename S>
+__global__ __launch_bounds__(kBlock) void narrow2_kernel(const float *from0, S *to0, int64_t count0,
+                                                         const float *from1, S *to1,
+                                                         int64_t count1) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < count0; k += stride)
+    Storage<S>::store(to0 + k, from0[k]);
+  for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < count1; k += stride)
+    Storage<S>::store(to1 + k, from1[k]);
 }
 
 template <typename R>
@@ -253,6 +272,28 @@ hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
   return hipGetLastError();
 }
 
+hipError_t ZeroRanges::launch(hipStream_t stream) const {
+  if (count == 0) return hipSuccess;
+  size_t most = 0;
+  for (int i = 0; i < count; ++i) most = bytes[i] > most ? bytes[i] : most;
+  fill_zero_ranges_kernel<<<grid_for((int64_t)(most / 16 + 32), kBlock), kBlock, 0, stream>>>(*this);
+  return hipGetLastError();
+}
+
+template <typename S>
+hipError_t launch_narrow2(const float *from0, S *to0, int64_t count0, const float *from1, S *to1,
+                          int64_t count1, hipStream_t stream) {
+  const int64_t most = count0 > count1 ? count0 : count1;
+  if (most == 0) return hipSuccess;
+  narrow2_kernel<S><<<grid_for(most, kBlock), kBlock, 0, stream>>>(from0, to0, count0, from1, to1,
+                                                                  count1);
+  return hipGetLastError();
+}
+template hipError_t launch_narrow2<__half>(const float *, __half *, int64_t, const float *, __half *,
+                                           int64_t, hipStream_t);
+template hipError_t launch_narrow2<bf16_t>(const float *, bf16_t *, int64_t, const float *, bf16_t *,
+                                           int64_t, hipStream_t);
+
 template <typename S>
 hipError_t launch_narrow(const float *from, S *to, int64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
@@ -293,16 +334,16 @@ hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream) {
   const int64_t n_src = a.B * a.N * a.srcH * a.srcW * a.C;
   const int64_t n_depth = a.depth_grid ? a.voxels() : a.pixels();
   hipError_t err;
+  ZeroRanges zero;  // everything the kernel accumulates into, one launch
   if (Is16<S>::value) {
-    if ((err = launch_fill_zero(a.ref_grad_acc, (size_t)n_ref * 4, stream)) != hipSuccess) return err;
-    if ((err = launch_fill_zero(a.src_grad_acc, (size_t)n_src * 4, stream)) != hipSuccess) return err;
+    zero.add(a.ref_grad_acc, (size_t)n_ref * 4);
+    zero.add(a.src_grad_acc, (size_t)n_src * 4);
   } else {
-    if ((err = launch_fill_zero(a.ref_grad, (size_t)n_ref * sizeof(S), stream)) != hipSuccess) return err;
-    if ((err = launch_fill_zero(a.src_grad, (size_t)n_src * sizeof(S), stream)) != hipSuccess) return err;
+    zero.add(a.ref_grad, (size_t)n_ref * sizeof(S));
+    zero.add(a.src_grad, (size_t)n_src * sizeof(S));
   }
-  if (a.depth_grad != nullptr &&
-      (err = launch_fill_zero(a.depth_grad, (size_t)n_depth * sizeof(R), stream)) != hipSuccess)
-    return err;
+  if (a.depth_grad != nullptr) zero.add(a.depth_grad, (size_t)n_depth * sizeof(R));
+  if ((err = zero.launch(stream)) != hipSuccess) return err;
   const int64_t total = a.voxels() * a.C;
   if (total > 0) {
     const int grid = grid_for(total, kBlock);
@@ -325,8 +366,9 @@ hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream) {
     if ((err = hipGetLastError()) != hipSuccess) return err;
   }
   if constexpr (Is16<S>::value) {
-    if ((err = launch_narrow<S>(a.ref_grad_acc, a.ref_grad, n_ref, stream)) != hipSuccess) return err;
-    if ((err = launch_narrow<S>(a.src_grad_acc, a.src_grad, n_src, stream)) != hipSuccess) return err;
+    if ((err = launch_narrow2<S>(a.ref_grad_acc, a.ref_grad, n_ref, a.src_grad_acc, a.src_grad, n_src,
+                                 stream)) != hipSuccess)
+      return err;
   }
   return hipSuccess;
 }

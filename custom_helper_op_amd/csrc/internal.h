@@ -138,8 +138,26 @@ hipError_t launch_tiled_backward_wide(const Args<S> &a, hipStream_t stream);
 
 // Utility launches.
 hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
+// Up to three ranges zeroed by ONE launch (a launch costs ~5 us, the ranges are small):
+// collect them with add(), then launch().
+struct ZeroRanges {
+  unsigned char *ptr[3] = {nullptr, nullptr, nullptr};
+  size_t bytes[3] = {0, 0, 0};
+  int count = 0;
+  void add(void *p, size_t n) {
+    if (n == 0) return;
+    ptr[count] = static_cast<unsigned char *>(p);
+    bytes[count] = n;
+    ++count;
+  }
+  hipError_t launch(hipStream_t stream) const;
+};
 template <typename S>
 hipError_t launch_narrow(const float *from, S *to, int64_t count, hipStream_t stream);
+// two fp32 images narrowed to 16-bit storage by one launch
+template <typename S>
+hipError_t launch_narrow2(const float *from0, S *to0, int64_t count0, const float *from1, S *to1,
+                          int64_t count1, hipStream_t stream);
 
 template <typename R>
 hipError_t launch_sample_coords(R half, int64_t B, int64_t H, int64_t W, int64_t D, int64_t N,

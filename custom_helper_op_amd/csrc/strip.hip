@@ -502,13 +502,14 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
   void *src_img = sizeof(S) == 2 ? (void *)a.src_grad_acc : (void *)a.src_grad;
   void *ref_img = sizeof(S) == 2 ? (void *)a.ref_grad_acc : (void *)a.ref_grad;
   const size_t acc_size = sizeof(S) == 2 ? 4 : sizeof(S);
-  if ((err = launch_fill_zero(src_img, (size_t)n_src * acc_size, stream)) != hipSuccess) return err;
+  ZeroRanges zero;  // one launch for all of them
+  zero.add(src_img, (size_t)n_src * acc_size);
   if (g.nseg > 1) {
-    if ((err = launch_fill_zero(ref_img, (size_t)n_ref * acc_size, stream)) != hipSuccess) return err;
-    if (a.depth_grid == nullptr && a.depth_grad != nullptr &&
-        (err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(R), stream)) != hipSuccess)
-      return err;
+    zero.add(ref_img, (size_t)n_ref * acc_size);
+    if (a.depth_grid == nullptr && a.depth_grad != nullptr)
+      zero.add(a.depth_grad, (size_t)a.pixels() * sizeof(R));
   }
+  if ((err = zero.launch(stream)) != hipSuccess) return err;
   const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB) +
                       (g.carry ? strip_run_bytes<S>(a.N) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
@@ -525,8 +526,9 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
   }
   if ((err = hipGetLastError()) != hipSuccess) return err;
   if constexpr (sizeof(S) == 2) {
-    if ((err = launch_narrow<S>(a.ref_grad_acc, a.ref_grad, n_ref, stream)) != hipSuccess) return err;
-    if ((err = launch_narrow<S>(a.src_grad_acc, a.src_grad, n_src, stream)) != hipSuccess) return err;
+    if ((err = launch_narrow2<S>(a.ref_grad_acc, a.ref_grad, n_ref, a.src_grad_acc, a.src_grad, n_src,
+                                 stream)) != hipSuccess)
+      return err;
   }
   return hipSuccess;
 }

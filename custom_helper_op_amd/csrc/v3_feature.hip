@@ -368,13 +368,11 @@ hipError_t launch_v3_forward(const Args<S> &a, hipStream_t stream) {
 template <typename S>
 hipError_t launch_v3_backward(const Args<S> &a, hipStream_t stream) {
   hipError_t err;
-  if ((err = launch_fill_zero(a.ref_grad, (size_t)(a.pixels() * a.C) * sizeof(S), stream)) != hipSuccess)
-    return err;
-  if ((err = launch_fill_zero(a.src_grad, (size_t)(a.B * a.N * a.srcH * a.srcW * a.C) * sizeof(S),
-                              stream)) != hipSuccess)
-    return err;
-  if ((err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(S), stream)) != hipSuccess)
-    return err;
+  ZeroRanges zero;  // one launch
+  zero.add(a.ref_grad, (size_t)(a.pixels() * a.C) * sizeof(S));
+  zero.add(a.src_grad, (size_t)(a.B * a.N * a.srcH * a.srcW * a.C) * sizeof(S));
+  zero.add(a.depth_grad, (size_t)a.pixels() * sizeof(S));
+  if ((err = zero.launch(stream)) != hipSuccess) return err;
   const int64_t total = a.voxels();
   if (total == 0 || a.C == 0) return hipSuccess;
   const int grid = grid_for(total, kBlock);
@@ -411,11 +409,10 @@ hipError_t launch_feature_forward(const Args<S> &a, hipStream_t stream) {
 template <typename S>
 hipError_t launch_feature_backward(const Args<S> &a, hipStream_t stream) {
   hipError_t err;
-  if ((err = launch_fill_zero(a.src_grad, (size_t)(a.B * a.N * a.srcH * a.srcW * a.C) * sizeof(S),
-                              stream)) != hipSuccess)
-    return err;
-  if ((err = launch_fill_zero(a.depth_grad, (size_t)a.pixels() * sizeof(S), stream)) != hipSuccess)
-    return err;
+  ZeroRanges zero;  // one launch
+  zero.add(a.src_grad, (size_t)(a.B * a.N * a.srcH * a.srcW * a.C) * sizeof(S));
+  zero.add(a.depth_grad, (size_t)a.pixels() * sizeof(S));
+  if ((err = zero.launch(stream)) != hipSuccess) return err;
   constexpr int kVec = 16 / (int)sizeof(S);
   const bool wide = a.C % kVec == 0 && aligned16<S>(a.src) && aligned16<S>(a.cost_grad);
   const int64_t total = a.voxels() * a.N * (wide ? a.C / kVec : a.C);
