@@ -126,7 +126,8 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
   const R dflt = fill ? *a.default_cost : R(0);
   const int64_t row_step = (int64_t)srcW * C;
   StripRecords<R> rec = strip_records<R, 4>(smem, ppw * g.vg * kDB);
-  R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw * g.vg * kDB)) - 64;  // CORR: products of a pixel
+  // CORR: the products of a pixel's channels
+  R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw * g.vg * kDB)) - 64;
 
   for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
     R acc[kDB];
@@ -138,70 +139,70 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
       kcnt[jj] = 0;
     }
     for (int n0 = 0; n0 < N; n0 += g.vg) {
-    const int nv = min(g.vg, N - n0);
-    strip_sync();  // the records of the views before have been read
-    for (int item = cl; item < nv * kDB; item += lpp) {
-      const int nl = item / kDB, j = item - nl * kDB;
-      const int64_t cam = (int64_t)px.b * N + n0 + nl;
-      const int d = d0 + j;
-      int off = -1;
-      Sample<R> s;
-      s.k00 = s.k01 = s.k11 = s.k10 = R(0);
-      if (d < d_hi) {
-        const R depth = a.depth_grid ? a.depth_grid[px.pix * D + d]
-                                     : base + a.offsets[(int64_t)px.b * D + d];
-        project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
-        if (s.state == 2) off = (s.fh * srcW + s.fw) * C;
+      const int nv = min(g.vg, N - n0);
+      strip_sync();  // the records of the views before have been read
+      for (int item = cl; item < nv * kDB; item += lpp) {
+        const int nl = item / kDB, j = item - nl * kDB;
+        const int64_t cam = (int64_t)px.b * N + n0 + nl;
+        const int d = d0 + j;
+        int off = -1;
+        Sample<R> s;
+        s.k00 = s.k01 = s.k11 = s.k10 = R(0);
+        if (d < d_hi) {
+          const R depth = a.depth_grid ? a.depth_grid[px.pix * D + d]
+                                       : base + a.offsets[(int64_t)px.b * D + d];
+          project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
+          if (s.state == 2) off = (s.fh * srcW + s.fw) * C;
+        }
+        const int r = (nl * ppw + p) * kDB + j;
+        rec.off[r] = off;
+        rec.at(0, r) = s.k00;
+        rec.at(1, r) = s.k01;
+        rec.at(2, r) = s.k11;
+        rec.at(3, r) = s.k10;
       }
-      const int r = (nl * ppw + p) * kDB + j;
-      rec.off[r] = off;
-      rec.at(0, r) = s.k00;
-      rec.at(1, r) = s.k01;
-      rec.at(2, r) = s.k11;
-      rec.at(3, r) = s.k10;
-    }
-    strip_sync();
-    for (int nl = 0; nl < nv; ++nl) {
-      const int n = n0 + nl;
-      const int ridx = (nl * ppw + p) * kDB;
-      const int64_t cam = (int64_t)px.b * N + n;
-      const S *view = a.src + cam * srcH * srcW * C + (ch_ok ? cl : 0);
-      int cur = -1;
-      R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
+      strip_sync();
+      for (int nl = 0; nl < nv; ++nl) {
+        const int n = n0 + nl;
+        const int ridx = (nl * ppw + p) * kDB;
+        const int64_t cam = (int64_t)px.b * N + n;
+        const S *view = a.src + cam * srcH * srcW * C + (ch_ok ? cl : 0);
+        int cur = -1;
+        R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
 #pragma unroll
-      for (int jj = 0; jj < kDB; ++jj) {
-        const int off = rec.off[ridx + jj];
-        if (off < 0) continue;
-        if (off != cur) {
-          cur = off;
-          const S *q = view + off;
-          v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
-          v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
+        for (int jj = 0; jj < kDB; ++jj) {
+          const int off = rec.off[ridx + jj];
+          if (off < 0) continue;
+          if (off != cur) {
+            cur = off;
+            const S *q = view + off;
+            v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
+            v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
+          }
+          const R smp = rec.at(0, ridx + jj) * v00 + rec.at(1, ridx + jj) * v01 +
+                        rec.at(2, ridx + jj) * v11 + rec.at(3, ridx + jj) * v10;
+          R val;
+          if (CORR == 0) {
+            const R diff = smp - ref_c;
+            val = diff * diff;
+          } else {
+            // the group's products, added up from zero in channel order by the group's lane
+            s_prod[lane] = smp * ref_c;
+            strip_sync();
+            val = R(0);
+            if (cl < OC)
+              for (int c = 0; c < sub; ++c) val += s_prod[p * lpp + cl * sub + c];
+            strip_sync();
+          }
+          if (REDUCE == 0) {
+            acc[jj] += val;
+          } else if (CORR ? (acc[jj] < val) : (acc[jj] > val)) {
+            acc[jj] = val;
+            arg[jj] = n;
+          }
+          ++kcnt[jj];
         }
-        const R smp = rec.at(0, ridx + jj) * v00 + rec.at(1, ridx + jj) * v01 +
-                      rec.at(2, ridx + jj) * v11 + rec.at(3, ridx + jj) * v10;
-        R val;
-        if (CORR == 0) {
-          const R diff = smp - ref_c;
-          val = diff * diff;
-        } else {
-          // the group's products, added up from zero in channel order by the group's lane
-          s_prod[lane] = smp * ref_c;
-          strip_sync();
-          val = R(0);
-          if (cl < OC)
-            for (int c = 0; c < sub; ++c) val += s_prod[p * lpp + cl * sub + c];
-          strip_sync();
-        }
-        if (REDUCE == 0) {
-          acc[jj] += val;
-        } else if (CORR ? (acc[jj] < val) : (acc[jj] > val)) {
-          acc[jj] = val;
-          arg[jj] = n;
-        }
-        ++kcnt[jj];
       }
-    }
     }  // group of views
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) {
@@ -267,10 +268,9 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) dvox[jj] = R(0);
     for (int n0 = 0; n0 < N; n0 += g.vg) {
-    const int nv = min(g.vg, N - n0);
-    strip_sync();
-    for (int item = cl; item < nv * kDB; item += lpp) {
-      {
+      const int nv = min(g.vg, N - n0);
+      strip_sync();
+      for (int item = cl; item < nv * kDB; item += lpp) {
         const int nl = item / kDB, j = item - nl * kDB;
         const int64_t cam = (int64_t)px.b * N + n0 + nl;
         const int ridx = (nl * ppw + p) * kDB;
@@ -306,89 +306,88 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         rec.at(7, ridx + j) = fw;
         rec.at(8, ridx + j) = cnt;
       }
-    }
-    strip_sync();
-    for (int nl = 0; nl < nv; ++nl) {
-      const int n = n0 + nl;
-      const int ridx = (nl * ppw + p) * kDB;
-      const int64_t view_off = ((int64_t)px.b * N + n) * srcH * srcW * C + (ch_ok ? cl : 0);
-      const S *view = a.src + view_off;
-      Acc *gview = src_grad + view_off;
-      int cur = -1, have = -1;  // cell of the open run, cell whose taps are in registers
-      R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
-      R g00 = R(0), g01 = R(0), g11 = R(0), g10 = R(0);
-      if (carry) {
-        cur = s_cur[n * 64 + lane];
-        g00 = s_run[(n * 4 + 0) * 64 + lane], g01 = s_run[(n * 4 + 1) * 64 + lane];
-        g11 = s_run[(n * 4 + 2) * 64 + lane], g10 = s_run[(n * 4 + 3) * 64 + lane];
-      }
-      auto flush = [&]() {
-        if (cur >= 0 && ch_ok) {
-          Acc *q = gview + cur;
-          if (g00 != R(0)) atomic_add(q, (Acc)g00);
-          if (g01 != R(0)) atomic_add(q + C, (Acc)g01);
-          if (g11 != R(0)) atomic_add(q + C + row_step, (Acc)g11);
-          if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
+      strip_sync();
+      for (int nl = 0; nl < nv; ++nl) {
+        const int n = n0 + nl;
+        const int ridx = (nl * ppw + p) * kDB;
+        const int64_t view_off = ((int64_t)px.b * N + n) * srcH * srcW * C + (ch_ok ? cl : 0);
+        const S *view = a.src + view_off;
+        Acc *gview = src_grad + view_off;
+        int cur = -1, have = -1;  // cell of the open run, cell whose taps are in registers
+        R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
+        R g00 = R(0), g01 = R(0), g11 = R(0), g10 = R(0);
+        if (carry) {
+          cur = s_cur[n * 64 + lane];
+          g00 = s_run[(n * 4 + 0) * 64 + lane], g01 = s_run[(n * 4 + 1) * 64 + lane];
+          g11 = s_run[(n * 4 + 2) * 64 + lane], g10 = s_run[(n * 4 + 3) * 64 + lane];
         }
-        g00 = g01 = g11 = g10 = R(0);
-      };
+        auto flush = [&]() {
+          if (cur >= 0 && ch_ok) {
+            Acc *q = gview + cur;
+            if (g00 != R(0)) atomic_add(q, (Acc)g00);
+            if (g01 != R(0)) atomic_add(q + C, (Acc)g01);
+            if (g11 != R(0)) atomic_add(q + C + row_step, (Acc)g11);
+            if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
+          }
+          g00 = g01 = g11 = g10 = R(0);
+        };
 #pragma unroll
-      for (int jj = 0; jj < kDB; ++jj) {
-        const int off = rec.off[ridx + jj];
-        if (off < 0) continue;
-        const int64_t i = px.pix * D + d0 + jj;
-        if (off != cur) {
-          flush();
-          cur = off;
+        for (int jj = 0; jj < kDB; ++jj) {
+          const int off = rec.off[ridx + jj];
+          if (off < 0) continue;
+          const int64_t i = px.pix * D + d0 + jj;
+          if (off != cur) {
+            flush();
+            cur = off;
+          }
+          if (off != have) {
+            have = off;
+            const S *q = view + off;
+            v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
+            v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
+          }
+          if (!ch_ok) continue;
+          if (REDUCE != 0 && a.mask_in[i * OC + oc] != n) continue;  // another view won (:553)
+          const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
+                  k10 = rec.at(3, ridx + jj);
+          const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
+          const R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
+          // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
+          // reference's division (one division per voxel in phase 1 instead of one per element)
+          const R inv = rec.at(8, ridx + jj);
+          R gv;
+          if (CORR == 0) {
+            const R diff = smp - ref_c;
+            gv = REDUCE == 0 ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
+            racc += -gv;
+          } else {
+            gv = REDUCE == 0 ? cg * inv : cg;  // v2 :461, :583
+            racc += gv * smp;
+            gv = gv * ref_c;
+          }
+          g00 += gv * k00;
+          g01 += gv * k01;
+          g11 += gv * k11;
+          g10 += gv * k10;
+          if (want_depth) {
+            const R t1 = v11 - v10 - v01 + v00;
+            const R h_grad = gv * (t1 * rec.at(5, ridx + jj) + v10 - v00);
+            const R w_grad = gv * (t1 * rec.at(4, ridx + jj) + v01 - v00);
+            const R dl = rec.at(6, ridx + jj) * h_grad + rec.at(7, ridx + jj) * w_grad;
+            if (per_voxel)
+              dvox[jj] += dl;
+            else
+              dpart += dl;
+          }
         }
-        if (off != have) {
-          have = off;
-          const S *q = view + off;
-          v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
-          v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
-        }
-        if (!ch_ok) continue;
-        if (REDUCE != 0 && a.mask_in[i * OC + oc] != n) continue;  // another view won (:553)
-        const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
-                k10 = rec.at(3, ridx + jj);
-        const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
-        const R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
-        // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
-        // reference's division (one division per voxel in phase 1 instead of one per element)
-        const R inv = rec.at(8, ridx + jj);
-        R gv;
-        if (CORR == 0) {
-          const R diff = smp - ref_c;
-          gv = REDUCE == 0 ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
-          racc += -gv;
+        if (carry) {
+          s_cur[n * 64 + lane] = cur;
+          s_run[(n * 4 + 0) * 64 + lane] = g00, s_run[(n * 4 + 1) * 64 + lane] = g01;
+          s_run[(n * 4 + 2) * 64 + lane] = g11, s_run[(n * 4 + 3) * 64 + lane] = g10;
         } else {
-          gv = REDUCE == 0 ? cg * inv : cg;  // v2 :461, :583
-          racc += gv * smp;
-          gv = gv * ref_c;
-        }
-        g00 += gv * k00;
-        g01 += gv * k01;
-        g11 += gv * k11;
-        g10 += gv * k10;
-        if (want_depth) {
-          const R t1 = v11 - v10 - v01 + v00;
-          const R h_grad = gv * (t1 * rec.at(5, ridx + jj) + v10 - v00);
-          const R w_grad = gv * (t1 * rec.at(4, ridx + jj) + v01 - v00);
-          const R dl = rec.at(6, ridx + jj) * h_grad + rec.at(7, ridx + jj) * w_grad;
-          if (per_voxel)
-            dvox[jj] += dl;
-          else
-            dpart += dl;
+          flush();
         }
       }
-      if (carry) {
-        s_cur[n * 64 + lane] = cur;
-        s_run[(n * 4 + 0) * 64 + lane] = g00, s_run[(n * 4 + 1) * 64 + lane] = g01;
-        s_run[(n * 4 + 2) * 64 + lane] = g11, s_run[(n * 4 + 3) * 64 + lane] = g10;
-      } else {
-        flush();
-      }
-    }
     }  // group of views
     if (per_voxel && want_depth) {
 #pragma unroll

@@ -1,7 +1,8 @@
-// Tiled cost-volume kernels for gfx950 (MEAN reduce).
+// Tiled cost-volume kernels for gfx950 (MEAN and MIN / MAX reduces, every op of the family).
 //
-// Work decomposition.  A workgroup is one wavefront.  It owns PPW = 64/LPP consecutive
-// pixels of one image and one contiguous segment of the D depth hypotheses; the LPP lanes
+// Work decomposition.  A workgroup is one wavefront.  It owns PPW = 64/LPP pixels of one
+// image (two rows of PPW/2: a compact tile's samples change their texel cell together more
+// often than a long row's) and one contiguous segment of the D depth hypotheses; the LPP lanes
 // of a pixel each own VEC consecutive channels (C = LPP*VEC), so every tap read and every
 // cost-row write of a pixel is one contiguous C*sizeof(S) segment.  Depth runs innermost:
 // along the walk the sample point of a view slides along an epipolar line by a fraction of
