@@ -90,9 +90,9 @@ class Runner:
                                                      p(self.Rs), p(self.Ts), p(self.cost),
                                                      p(self.mask))
         elif self.agg:
-            rc = lib.chop_cost_aggregate_fwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
-                                                 p(self.base_plane), p(self.offsets), p(self.Rs),
-                                                 p(self.Ts), p(self.cost), p(self.mask))
+            fn = lib.chop_cost_aggregate_fwd_f64 if self.f64 else lib.chop_cost_aggregate_fwd_f32
+            rc = fn(s, self.red, 1, *self.dims, p(self.ref), p(self.src), p(self.base_plane),
+                    p(self.offsets), p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
         elif self.v3:
             rc = lib.chop_cost_volume_v3_fwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
                                                  p(self.ref), p(self.src), p(self.base_plane),
@@ -133,9 +133,9 @@ class Runner:
                                                      p(self.ref), p(self.src), p(self.depth_grid),
                                                      p(self.Rs), p(self.Ts), *tail)
         elif self.agg:
-            rc = lib.chop_cost_aggregate_bwd_f32(s, self.red, 1, *self.dims, p(self.ref), p(self.src),
-                                                 p(self.base_plane), p(self.offsets), p(self.Rs),
-                                                 p(self.Ts), *tail)
+            fn = lib.chop_cost_aggregate_bwd_f64 if self.f64 else lib.chop_cost_aggregate_bwd_f32
+            rc = fn(s, self.red, 1, *self.dims, p(self.ref), p(self.src), p(self.base_plane),
+                    p(self.offsets), p(self.Rs), p(self.Ts), *tail)
         elif self.v3:
             rc = lib.chop_cost_volume_v3_bwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
                                                  p(self.ref), p(self.src), p(self.base_plane),
@@ -347,8 +347,9 @@ def main():
     wl = make_workload(a.workload, with_cost_grad=False)
     wl.reduce_method = a.reduce
     if a.float64 or a.channels:
-        if wl.op != "v1" or wl.storage != "f32" or a.aggregate or a.v3 or a.feature:
-            sys.exit("bench.py: --float64 / --channels need a float32 CostVolume workload (1, 2 or 5)")
+        if wl.op != "v1" or wl.storage != "f32" or a.v3 or a.feature:
+            sys.exit("bench.py: --float64 / --channels need a float32 CostVolume workload (1, 2 or 5), "
+                     "alone or with --aggregate")
         if a.channels:
             if not 1 <= a.channels <= wl.C:
                 sys.exit("bench.py: --channels must be 1..%d for this workload" % wl.C)
@@ -359,7 +360,7 @@ def main():
         if a.float64:
             wl.storage = "f64"
     if a.aggregate:
-        if wl.op != "v1" or wl.storage != "f32":
+        if wl.op != "v1" or wl.storage not in ("f32", "f64"):
             sys.exit("bench.py: --aggregate needs a float32 CostVolume workload (1, 2 or 5)")
         wl.op = "agg"
     if a.v3 or a.feature:

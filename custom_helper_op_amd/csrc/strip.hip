@@ -1,7 +1,8 @@
 // Strip kernels: the wave-per-pixel-strip decomposition for every shape the tiled kernels do
 // not take -- float64 (the element type of the reference's own tests), channel counts that
 // are not 4 x a power of two (the reference tests use 3, 5 and 9), any number of views -- for
-// CostVolume and CostVolumeV2, both reduces, all four storage types, up to 64 channels.
+// CostVolume, CostVolumeV2 and CostAggregate, both reduces, all four storage types, up to 64
+// channels.
 //
 // A workgroup is one wavefront.  It owns 64/LPP consecutive pixels (LPP = the power of two
 // >= C: one lane per channel, so a tap read or a cost-row write of a pixel is one contiguous
@@ -115,8 +116,9 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
   const int64_t tile = (int64_t)blockIdx.x / g.nseg;
   const int segi = (int)((int64_t)blockIdx.x - tile * g.nseg);
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  const int OC = CORR ? a.groups : C;
-  const int sub = CORR ? C / a.groups : 1;
+  constexpr bool AGG = CORR == 2;  // CostAggregate: one value per voxel
+  const int OC = CORR == 1 ? a.groups : AGG ? 1 : C;
+  const int sub = CORR == 1 ? C / a.groups : 1;
   const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
   const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
   const bool ch_ok = cl < C, out_ok = px.ok && cl < OC;
@@ -126,15 +128,20 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
   const R dflt = fill ? *a.default_cost : R(0);
   const int64_t row_step = (int64_t)srcW * C;
   StripRecords<R> rec = strip_records<R, 4>(smem, ppw * g.vg * kDB);
-  // CORR: the products of a pixel's channels
+  // group correlation: the products of a pixel's channels
   R *s_prod = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(4, ppw * g.vg * kDB)) - 64;
+  // CostAggregate: the chunk's squared differences, one row of 64 lanes per depth.  Lane
+  // (jj mod LPP) of a pixel owns voxel (pixel, d0 + jj): it adds the row up in channel order,
+  // which is the order of the reference's scalar loop (cost_aggregate_kernels_gpu.cu.cc:
+  // 108-113, :206-216), so the sums and the winning views are the oracle's to the bit.
+  R *s_rows = s_prod + 64;
 
   for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
     R acc[kDB];
     int arg[kDB], kcnt[kDB];
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) {
-      acc[jj] = REDUCE == 0 ? R(0) : (CORR ? Limits<R>::min_positive() : Limits<R>::max());
+      acc[jj] = REDUCE == 0 ? R(0) : (CORR == 1 ? Limits<R>::min_positive() : Limits<R>::max());
       arg[jj] = -1;
       kcnt[jj] = 0;
     }
@@ -182,9 +189,13 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
           const R smp = rec.at(0, ridx + jj) * v00 + rec.at(1, ridx + jj) * v01 +
                         rec.at(2, ridx + jj) * v11 + rec.at(3, ridx + jj) * v10;
           R val;
-          if (CORR == 0) {
+          if (CORR != 1) {
             const R diff = smp - ref_c;
             val = diff * diff;
+            if constexpr (AGG) {
+              s_rows[jj * 64 + lane] = val;
+              continue;
+            }
           } else {
             // the group's products, added up from zero in channel order by the group's lane
             s_prod[lane] = smp * ref_c;
@@ -196,14 +207,58 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
           }
           if (REDUCE == 0) {
             acc[jj] += val;
-          } else if (CORR ? (acc[jj] < val) : (acc[jj] > val)) {
+          } else if (CORR == 1 ? (acc[jj] < val) : (acc[jj] > val)) {
             acc[jj] = val;
             arg[jj] = n;
           }
           ++kcnt[jj];
         }
+        if constexpr (AGG) {
+          strip_sync();  // the rows are written
+          // the owners work side by side: lane cl owns depths cl, cl + LPP, ... of its pixel
+          // (acc / kcnt / arg are indexed by k, the k-th depth a lane owns)
+#pragma unroll
+          for (int k = 0; k < kDB; ++k) {
+            const int jj = cl + k * lpp;
+            if (jj >= kDB || rec.off[ridx + jj] < 0) continue;
+            const R *row = s_rows + jj * 64 + p * lpp;
+            // eight LDS reads in flight, then eight additions in channel order
+            R sum = REDUCE == 0 ? acc[k] : R(0);
+            for (int c0 = 0; c0 < C; c0 += 8) {
+              R v[8];
+#pragma unroll
+              for (int u = 0; u < 8; ++u) v[u] = row[min(c0 + u, C - 1)];
+#pragma unroll
+              for (int u = 0; u < 8; ++u)
+                if (c0 + u < C) sum += v[u];
+            }
+            if (REDUCE == 0) {
+              acc[k] = sum;
+              ++kcnt[k];
+            } else if (acc[k] > sum) {
+              acc[k] = sum, arg[k] = n;  // strict: the earliest view keeps a tie
+            }
+          }
+          strip_sync();  // ... and read, before the next view overwrites them
+        }
       }
     }  // group of views
+    if constexpr (AGG) {
+#pragma unroll
+      for (int k = 0; k < kDB; ++k) {
+        const int jj = cl + k * lpp, d = d0 + jj;
+        if (jj >= kDB || d >= d_hi || !px.ok) continue;
+        const int64_t i = px.pix * D + d;
+        const bool any = REDUCE == 0 ? kcnt[k] > 0 : arg[k] >= 0;
+        // :118-123 cost / (T)(used * channels), :222-227 cost / (T)channels
+        R out = REDUCE == 0 ? acc[k] / static_cast<R>((int64_t)kcnt[k] * C)
+                            : acc[k] / static_cast<R>(C);
+        if (!any) out = fill ? dflt : R(0);
+        a.mask[i] = REDUCE == 0 ? kcnt[k] : arg[k];
+        Storage<S>::store(a.cost + i, out);
+      }
+      continue;
+    }
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) {
       const int d = d0 + jj;
@@ -242,17 +297,19 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   const int64_t tile = (int64_t)blockIdx.x / g.nseg;
   const int segi = (int)((int64_t)blockIdx.x - tile * g.nseg);
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  const int OC = CORR ? a.groups : C;
-  const int sub = CORR ? C / a.groups : 1;
+  constexpr bool AGG = CORR == 2;  // CostAggregate: one upstream value per voxel
+  const int OC = CORR == 1 ? a.groups : AGG ? 1 : C;
+  const int sub = CORR == 1 ? C / a.groups : 1;
   const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
   const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
   const bool ch_ok = cl < C && px.ok;
-  const int oc = CORR ? (ch_ok ? cl / sub : 0) : (ch_ok ? cl : 0);
+  const int oc = CORR == 1 ? (ch_ok ? cl / sub : 0) : AGG ? 0 : (ch_ok ? cl : 0);
   const R ref_c = ch_ok ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
   const bool per_voxel = a.depth_grid != nullptr, want_depth = a.depth_grad != nullptr;
   const int64_t row_step = (int64_t)srcW * C;
   // fields: the four weights, dh, dw, the two depth-chain factors, 1 / view count
+  // (CostAggregate: 1 / (view count * channels), or 1 / channels for the MIN reduce)
   StripRecords<R> rec = strip_records<R, 9>(smem, ppw * g.vg * kDB);
   // open runs between two chunks: per view the cell and its four tap sums, one slot per lane
   // (a lane only ever reads its own slots back)
@@ -291,7 +348,10 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
               const R zz = s.z * s.z;
               fh = (s.h_coef * s.z - s.z_coef * s.h3d) / zz;
               fw = (s.w_coef * s.z - s.z_coef * s.w3d) / zz;
-              cnt = R(1) / static_cast<R>(m0);
+              if constexpr (AGG)  // cost_aggregate_kernels_gpu.cu.cc:388, :502
+                cnt = R(1) / static_cast<R>(REDUCE == 0 ? (int64_t)m0 * C : (int64_t)C);
+              else
+                cnt = R(1) / static_cast<R>(m0);
             }
           }
         }
@@ -356,9 +416,9 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
           // reference's division (one division per voxel in phase 1 instead of one per element)
           const R inv = rec.at(8, ridx + jj);
           R gv;
-          if (CORR == 0) {
+          if (CORR != 1) {
             const R diff = smp - ref_c;
-            gv = REDUCE == 0 ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
+            gv = (REDUCE == 0 || AGG) ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
             racc += -gv;
           } else {
             gv = REDUCE == 0 ? cg * inv : cg;  // v2 :461, :583
@@ -460,7 +520,9 @@ StripGeom strip_geometry(const Args<S> &a) {
 
 template <typename S>
 bool strip_supported(const Args<S> &a) {
-  if (a.corr != SQUARED_DIFFERENCE && a.corr != GROUP_CORRELATION) return false;
+  if (a.corr != SQUARED_DIFFERENCE && a.corr != GROUP_CORRELATION &&
+      a.corr != SUM_SQUARED_DIFFERENCE)
+    return false;
   if (a.C < 1 || a.C > 64 || a.N < 1 || a.D < 1 || a.pixels() < 1) return false;
   if (a.corr == GROUP_CORRELATION && (a.groups < 1 || a.C % a.groups != 0)) return false;
   if (a.srcH < 2 || a.srcW < 2) return false;                   // no sample can be accepted
@@ -473,9 +535,16 @@ template <typename S>
 hipError_t launch_strip_forward(const Args<S> &a, hipStream_t stream) {
   using R = typename Storage<S>::Real;
   const StripGeom g = strip_geometry(a);
-  const size_t smem = strip_lds_bytes<R>(4, (64 >> g.lpp_shift) * g.vg * kDB);
+  // CostAggregate adds one row of 64 values per depth of a chunk
+  const size_t smem = strip_lds_bytes<R>(4, (64 >> g.lpp_shift) * g.vg * kDB) +
+                      (a.corr == SUM_SQUARED_DIFFERENCE ? (size_t)kDB * 64 * sizeof(R) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
-  if (a.corr == SQUARED_DIFFERENCE) {
+  if (a.corr == SUM_SQUARED_DIFFERENCE) {
+    if (a.reduce == 0)
+      strip_forward_kernel<S, 2, 0><<<grid, block, smem, stream>>>(a, g);
+    else
+      strip_forward_kernel<S, 2, 1><<<grid, block, smem, stream>>>(a, g);
+  } else if (a.corr == SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
       strip_forward_kernel<S, 0, 0><<<grid, block, smem, stream>>>(a, g);
     else
@@ -512,7 +581,12 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
   const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB) +
                       (g.carry ? strip_run_bytes<S>(a.N) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
-  if (a.corr == SQUARED_DIFFERENCE) {
+  if (a.corr == SUM_SQUARED_DIFFERENCE) {
+    if (a.reduce == 0)
+      strip_backward_kernel<S, 2, 0><<<grid, block, smem, stream>>>(a, g);
+    else
+      strip_backward_kernel<S, 2, 1><<<grid, block, smem, stream>>>(a, g);
+  } else if (a.corr == SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
       strip_backward_kernel<S, 0, 0><<<grid, block, smem, stream>>>(a, g);
     else

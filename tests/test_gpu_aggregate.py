@@ -11,7 +11,7 @@ from gpu_util import assert_backward_close, assert_forward_close, dev, host
 
 pytestmark = pytest.mark.gpu
 
-FAMILIES = [pytest.param(1, id="general"), pytest.param(0, id="auto")]
+FAMILIES = [pytest.param(1, id="general"), pytest.param(2, id="strip"), pytest.param(0, id="auto")]
 # (B, N, H, W, C, D): the reference tests' parameter sets plus channel counts the tiled
 # kernels take (multiples of 4) and ones they do not
 SHAPES = [(1, 1, 12, 16, 3, 5), (1, 2, 12, 16, 8, 9), (2, 2, 12, 18, 5, 10), (2, 3, 12, 16, 16, 6),
@@ -35,10 +35,13 @@ def _args(t):
 
 
 def _expect_family(family, C, reduce, dtype, backward=False):
-    """The tiled kernels take float32 with a channel count that is 4 times a power of two."""
-    tiled = family == 0 and dtype == np.float32 and C in (4, 8, 16, 32, 64)
+    """Which kernels served the last call (1 general, 2 tiled, 3 strip).  Left to itself the
+    library gives float32 with a channel count of 4 times a power of two to the tiled kernels
+    and everything else (float64, other channel counts) to the strip kernels."""
+    tiled = dtype == np.float32 and C in (4, 8, 16, 32, 64)
+    want = {1: 1, 2: 3, 0: 2 if tiled else 3}[family]
     got = _lib.load().chop_last_kernel_family()
-    assert got == (2 if tiled else 1), (got, family, C, reduce, dtype)
+    assert got == want, (got, want, family, C, reduce, dtype)
 
 
 @pytest.mark.parametrize("family", FAMILIES)
@@ -55,7 +58,7 @@ def test_forward(oracle, family, shape, reduce, dtype):
         _expect_family(family, C, reduce, dtype)
         assert cost.shape == (B, H, W, D) and mask.shape == (B, H, W, D)
         assert np.array_equal(host(mask), want_mask)
-        if _lib.load().chop_last_kernel_family() == 1 or reduce == "MIN":
+        if _lib.load().chop_last_kernel_family() != 2 or reduce == "MIN":
             assert np.array_equal(host(cost), want_cost)  # literal operation order: same bits
         else:
             assert_forward_close(host(cost), want_cost)

@@ -326,7 +326,7 @@ def test_backward_without_the_depth_gradient(oracle, family):
     acg = np.ascontiguousarray(t["cost_grad"][..., 0])
     want = oracle.cost_aggregate_bwd(*args, acg, amask)
     got = chop.cost_aggregate_grad(*_v1_inputs(t), dev(acg), dev(amask), need_depth_grad=False)
-    _assert_family(1 if family == 2 else family)  # no strip kernels for CostAggregate
+    _assert_family(family)
     assert got[2] is None
     assert_backward_close(host(got[0]), want[0])
     assert_backward_close(host(got[1]), want[1])

@@ -98,8 +98,8 @@ def test_random_shape_other_ops(oracle, seed):
     want_cost, want_mask = oracle.cost_aggregate_fwd(*args, reduce, half)
     cost, mask = chop.cost_aggregate_raw(*d_args, reduce, half)
     assert np.array_equal(host(mask), want_mask)
-    if lib.chop_last_kernel_family() == 1 or reduce == "MIN":
-        assert np.array_equal(host(cost), want_cost)
+    if lib.chop_last_kernel_family() != 2 or reduce == "MIN":
+        assert np.array_equal(host(cost), want_cost)  # general and strip kernels: bit-identical
     else:
         assert_forward_close(host(cost), want_cost)
     cg = rng.standard_normal(want_cost.shape).astype(dtype)
