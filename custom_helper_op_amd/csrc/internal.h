@@ -99,8 +99,9 @@ template <typename S>
 hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream);
 
 // Strip kernels: one wavefront per strip of pixels, one lane per channel, depth innermost.
-// CostVolume and CostVolumeV2 with up to 64 channels, any view count, all storage types:
-// what the tiled kernels decline (float64, channel counts other than 4 x 2^k) runs here.
+// CostVolume, CostVolumeV2 and CostAggregate with up to 64 channels, any view count, all
+// storage types: what the tiled kernels decline (float64, channel counts other than 4 x 2^k)
+// runs here.
 template <typename S>
 bool strip_supported(const Args<S> &a);
 template <typename S>
