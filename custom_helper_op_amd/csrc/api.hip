@@ -286,6 +286,11 @@ int feature_call(void *stream, int half_centor, const Dims &d, const S *src, con
                       : launch_status(launch_tiled_forward(a, s), "tiled FeatureAggregate forward launch");
     }
   }
+  if (g_kernel_family != 1 && work && strip_supported(a)) {
+    g_last_family = 3;
+    return backward ? launch_status(launch_strip_backward(a, s), "strip FeatureAggregate backward launch")
+                    : launch_status(launch_strip_forward(a, s), "strip FeatureAggregate forward launch");
+  }
   g_last_family = 1;
   if (backward) return launch_status(launch_feature_backward(a, s), "FeatureAggregate backward launch");
   return launch_status(launch_feature_forward(a, s), "FeatureAggregate forward launch");

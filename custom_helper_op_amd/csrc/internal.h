@@ -99,8 +99,8 @@ template <typename S>
 hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream);
 
 // Strip kernels: one wavefront per strip of pixels, one lane per channel, depth innermost.
-// CostVolume, CostVolumeV2 and CostAggregate with up to 64 channels, any view count, all
-// storage types: what the tiled kernels decline (float64, channel counts other than 4 x 2^k)
+// CostVolume, CostVolumeV2, CostAggregate and FeatureAggregate with up to 64 channels, any view
+// count, all storage types: what the tiled kernels decline (float64, channel counts other than 4 x 2^k)
 // runs here.
 template <typename S>
 bool strip_supported(const Args<S> &a);

@@ -1,8 +1,8 @@
 // Strip kernels: the wave-per-pixel-strip decomposition for every shape the tiled kernels do
 // not take -- float64 (the element type of the reference's own tests), channel counts that
 // are not 4 x a power of two (the reference tests use 3, 5 and 9), any number of views -- for
-// CostVolume, CostVolumeV2 and CostAggregate, both reduces, all four storage types, up to 64
-// channels.
+// CostVolume, CostVolumeV2, CostAggregate (both reduces) and FeatureAggregate, all four storage
+// types, up to 64 channels.
 //
 // A workgroup is one wavefront.  It owns 64/LPP consecutive pixels (LPP = the power of two
 // >= C: one lane per channel, so a tap read or a cost-row write of a pixel is one contiguous
@@ -116,13 +116,14 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
   const int64_t tile = (int64_t)blockIdx.x / g.nseg;
   const int segi = (int)((int64_t)blockIdx.x - tile * g.nseg);
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  constexpr bool AGG = CORR == 2;  // CostAggregate: one value per voxel
+  constexpr bool AGG = CORR == 2;   // CostAggregate: one value per voxel
+  constexpr bool FEAT = CORR == 4;  // FeatureAggregate: the samples themselves, a row per view
   const int OC = CORR == 1 ? a.groups : AGG ? 1 : C;
   const int sub = CORR == 1 ? C / a.groups : 1;
   const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
   const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
   const bool ch_ok = cl < C, out_ok = px.ok && cl < OC;
-  const R ref_c = ch_ok ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
+  const R ref_c = ch_ok && !FEAT ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
   const bool fill = a.default_cost != nullptr;  // the cost-map layers' default for empty voxels
   const R dflt = fill ? *a.default_cost : R(0);
@@ -179,6 +180,17 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
 #pragma unroll
         for (int jj = 0; jj < kDB; ++jj) {
           const int off = rec.off[ridx + jj];
+          if constexpr (FEAT) {
+            // zeros and a 0 in the mask for a view that is not accepted
+            // (feature_aggregate_kernels_gpu.cu.cc:114-118)
+            if (off < 0) {
+              const int64_t row = (px.pix * D + d0 + jj) * N + n;
+              if (d0 + jj < d_hi && px.ok) {
+                if (ch_ok) Storage<S>::store(a.cost + row * C + cl, R(0));
+                if (cl == 0) a.mask[row] = 0;
+              }
+            }
+          }
           if (off < 0) continue;
           if (off != cur) {
             cur = off;
@@ -188,6 +200,14 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
           }
           const R smp = rec.at(0, ridx + jj) * v00 + rec.at(1, ridx + jj) * v01 +
                         rec.at(2, ridx + jj) * v11 + rec.at(3, ridx + jj) * v10;
+          if constexpr (FEAT) {
+            const int64_t row = (px.pix * D + d0 + jj) * N + n;
+            if (px.ok) {  // (an accepted record implies d0 + jj < d_hi)
+              if (ch_ok) Storage<S>::store(a.cost + row * C + cl, smp);
+              if (cl == 0) a.mask[row] = 1;
+            }
+            continue;
+          }
           R val;
           if (CORR != 1) {
             const R diff = smp - ref_c;
@@ -243,6 +263,7 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
         }
       }
     }  // group of views
+    if constexpr (FEAT) continue;  // every row has been stored
     if constexpr (AGG) {
 #pragma unroll
       for (int k = 0; k < kDB; ++k) {
@@ -297,14 +318,15 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   const int64_t tile = (int64_t)blockIdx.x / g.nseg;
   const int segi = (int)((int64_t)blockIdx.x - tile * g.nseg);
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
-  constexpr bool AGG = CORR == 2;  // CostAggregate: one upstream value per voxel
+  constexpr bool AGG = CORR == 2;   // CostAggregate: one upstream value per voxel
+  constexpr bool FEAT = CORR == 4;  // FeatureAggregate: an upstream row and a mask entry per view
   const int OC = CORR == 1 ? a.groups : AGG ? 1 : C;
   const int sub = CORR == 1 ? C / a.groups : 1;
   const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
   const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
   const bool ch_ok = cl < C && px.ok;
   const int oc = CORR == 1 ? (ch_ok ? cl / sub : 0) : AGG ? 0 : (ch_ok ? cl : 0);
-  const R ref_c = ch_ok ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
+  const R ref_c = ch_ok && !FEAT ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
   const bool per_voxel = a.depth_grid != nullptr, want_depth = a.depth_grad != nullptr;
   const int64_t row_step = (int64_t)srcW * C;
@@ -338,7 +360,8 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         R fh = R(0), fw = R(0), cnt = R(1);
         if (d < d_hi && px.ok) {
           const int64_t i = px.pix * D + d;
-          const int32_t m0 = a.mask_in[REDUCE == 0 ? i : i * OC];
+          // FeatureAggregate: 1 / 0 per (voxel, view), :261-263
+          const int32_t m0 = FEAT ? a.mask_in[i * N + n0 + nl] : a.mask_in[REDUCE == 0 ? i : i * OC];
           // MEAN skips a voxel no view reached (:367), MIN one whose first entry is negative (:484)
           if (REDUCE == 0 ? (m0 > 0) : (m0 >= 0)) {
             const R depth = per_voxel ? a.depth_grid[i] : base + a.offsets[(int64_t)px.b * D + d];
@@ -348,7 +371,9 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
               const R zz = s.z * s.z;
               fh = (s.h_coef * s.z - s.z_coef * s.h3d) / zz;
               fw = (s.w_coef * s.z - s.z_coef * s.w3d) / zz;
-              if constexpr (AGG)  // cost_aggregate_kernels_gpu.cu.cc:388, :502
+              if constexpr (FEAT)
+                cnt = R(1);
+              else if constexpr (AGG)  // cost_aggregate_kernels_gpu.cu.cc:388, :502
                 cnt = R(1) / static_cast<R>(REDUCE == 0 ? (int64_t)m0 * C : (int64_t)C);
               else
                 cnt = R(1) / static_cast<R>(m0);
@@ -411,12 +436,15 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
           const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
                   k10 = rec.at(3, ridx + jj);
           const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
-          const R cg = Storage<S>::load(a.cost_grad + i * OC + oc);
+          const R cg = FEAT ? Storage<S>::load(a.cost_grad + (i * N + n) * C + cl)
+                            : Storage<S>::load(a.cost_grad + i * OC + oc);
           // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
           // reference's division (one division per voxel in phase 1 instead of one per element)
           const R inv = rec.at(8, ridx + jj);
           R gv;
-          if (CORR != 1) {
+          if constexpr (FEAT) {
+            gv = cg;  // feature_aggregate_kernels_gpu.cu.cc:307-311
+          } else if (CORR != 1) {
             const R diff = smp - ref_c;
             gv = (REDUCE == 0 || AGG) ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
             racc += -gv;
@@ -473,7 +501,7 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
       if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
     }
   }
-  if (ch_ok) {
+  if (ch_ok && !FEAT) {
     Acc *q = ref_grad + px.pix * C + cl;
     if (g.nseg == 1)
       *q = (Acc)racc;
@@ -521,7 +549,7 @@ StripGeom strip_geometry(const Args<S> &a) {
 template <typename S>
 bool strip_supported(const Args<S> &a) {
   if (a.corr != SQUARED_DIFFERENCE && a.corr != GROUP_CORRELATION &&
-      a.corr != SUM_SQUARED_DIFFERENCE)
+      a.corr != SUM_SQUARED_DIFFERENCE && a.corr != WARP_ONLY)
     return false;
   if (a.C < 1 || a.C > 64 || a.N < 1 || a.D < 1 || a.pixels() < 1) return false;
   if (a.corr == GROUP_CORRELATION && (a.groups < 1 || a.C % a.groups != 0)) return false;
@@ -539,7 +567,9 @@ hipError_t launch_strip_forward(const Args<S> &a, hipStream_t stream) {
   const size_t smem = strip_lds_bytes<R>(4, (64 >> g.lpp_shift) * g.vg * kDB) +
                       (a.corr == SUM_SQUARED_DIFFERENCE ? (size_t)kDB * 64 * sizeof(R) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
-  if (a.corr == SUM_SQUARED_DIFFERENCE) {
+  if (a.corr == WARP_ONLY) {
+    strip_forward_kernel<S, 4, 0><<<grid, block, smem, stream>>>(a, g);
+  } else if (a.corr == SUM_SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
       strip_forward_kernel<S, 2, 0><<<grid, block, smem, stream>>>(a, g);
     else
@@ -573,7 +603,7 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
   ZeroRanges zero;  // one launch for all of them
   zero.add(src_img, (size_t)n_src * acc_size);
   if (g.nseg > 1) {
-    zero.add(ref_img, (size_t)n_ref * acc_size);
+    if (a.corr != WARP_ONLY) zero.add(ref_img, (size_t)n_ref * acc_size);  // no reference image
     if (a.depth_grid == nullptr && a.depth_grad != nullptr)
       zero.add(a.depth_grad, (size_t)a.pixels() * sizeof(R));
   }
@@ -581,7 +611,9 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
   const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB) +
                       (g.carry ? strip_run_bytes<S>(a.N) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
-  if (a.corr == SUM_SQUARED_DIFFERENCE) {
+  if (a.corr == WARP_ONLY) {
+    strip_backward_kernel<S, 4, 0><<<grid, block, smem, stream>>>(a, g);
+  } else if (a.corr == SUM_SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
       strip_backward_kernel<S, 2, 0><<<grid, block, smem, stream>>>(a, g);
     else

@@ -274,11 +274,12 @@ def test_feature_backward(oracle, shape, dtype):
 
 @pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
 @pytest.mark.parametrize("N", [1, 3])
-@pytest.mark.parametrize("family", [pytest.param(1, id="general"), pytest.param(0, id="auto")])
+@pytest.mark.parametrize("family", [pytest.param(1, id="general"), pytest.param(2, id="strip"),
+                                    pytest.param(0, id="auto")])
 def test_feature_tiled_channel_widths(oracle, C, N, family):
     """Every lanes-per-pixel variant of the tiled kernels (C = 4 x a power of two, float32),
-    on an image whose pixel count is no multiple of the tile; the general kernels on the same
-    inputs for comparison.  Forward values are bit-identical in both families."""
+    on an image whose pixel count is no multiple of the tile; the general and the strip kernels
+    on the same inputs for comparison.  Forward values are bit-identical in all families."""
     lib = _lib.load()
     lib.chop_set_kernel_family(family)
     try:
@@ -286,13 +287,13 @@ def test_feature_tiled_channel_widths(oracle, C, N, family):
         t = reference_test_case(3, B, N, H, W, C, D, np.float32, seed=C + N)
         want, want_mask = oracle.feature_aggregate_fwd(*_args(t, FKEYS))
         mapped, mask = chop.feature_aggregate_raw(*_inputs(t, FKEYS))
-        assert lib.chop_last_kernel_family() == (2 if family == 0 else 1)
+        assert lib.chop_last_kernel_family() == {1: 1, 2: 3, 0: 2}[family]
         assert np.array_equal(host(mask), want_mask)
         assert np.array_equal(host(mapped), want)
         g = np.random.default_rng(C).normal(size=want.shape).astype(np.float32)
         want_g = oracle.feature_aggregate_bwd(*_args(t, FKEYS), g, want_mask)
         got_g = chop.feature_aggregate_grad(*_inputs(t, FKEYS), dev(g), mask)
-        assert lib.chop_last_kernel_family() == (2 if family == 0 else 1)
+        assert lib.chop_last_kernel_family() == {1: 1, 2: 3, 0: 2}[family]
         for a, b in zip(got_g, want_g):
             assert_backward_close(host(a), b)
     finally:
