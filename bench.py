@@ -30,6 +30,23 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 
+KERNEL_SOURCES = ("custom_helper_op_amd/csrc/tiled.h", "custom_helper_op_amd/csrc/tiled_launch.inc")
+
+
+def kernel_source_hashes():
+    """git blob hashes (sha1 of "blob <size>\\0" + content) of the sources of the tiled
+    kernels.  profiles/hbm_traffic.json records them beside the counters; bench.py reports
+    the traffic figure only while they still match (``python bench.py --print-kernel-hashes``
+    prints the current ones for that file)."""
+    import hashlib
+    out = {}
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            data = f.read()
+        out[rel] = hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+    return out
+
+
 class Runner:
     """Pre-allocated buffers + direct C-ABI calls, so a step enqueues kernels and nothing else."""
 
@@ -334,7 +351,12 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
+    ap.add_argument("--print-kernel-hashes", action="store_true",
+                    help="print the git blob hashes of the tiled kernels' sources and exit")
     a = ap.parse_args()
+    if a.print_kernel_hashes:
+        print(json.dumps({"kernel_sources": kernel_source_hashes()}, indent=2))
+        return
     if a.gpus != 1:
         sys.exit("bench.py: this operator runs on one GPU; --gpus %d is not supported "
                  "(there is no multi-GPU path to measure)" % a.gpus)
@@ -433,11 +455,17 @@ def main():
     achieved = d_b / (d_ms * 1e-3) / 1e9
     traffic = None
     traffic_source = None
+    traffic_stale = None
     try:  # HBM bytes per launch from rocprofv3 counters of a separate run of this command
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
             plain = wl.op in ("v1", "v2") and a.reduce == "MEAN" and not (a.float64 or a.channels)
-            t = json.load(f)[wl.name if plain and a.kernel_family == "auto" else "-"][dominant]
-        traffic = t["fetch_bytes"] + t["write_bytes"]
+            recorded = json.load(f)
+            t = recorded[wl.name if plain and a.kernel_family == "auto" else "-"][dominant]
+        # the counters belong to the kernel sources they were taken on: a figure measured on
+        # other sources is withheld, not reported
+        traffic_stale = recorded.get("kernel_sources") != kernel_source_hashes()
+        if not traffic_stale:
+            traffic = t["fetch_bytes"] + t["write_bytes"]
         traffic_source = "profiles/hbm_traffic.json (rocprofv3 FETCH_SIZE/WRITE_SIZE of a separate run)"
     except (OSError, KeyError, ValueError):
         pass
@@ -462,6 +490,7 @@ def main():
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "timing": "HIP events on the launch stream, caches overwritten before each call, median",
                      "traffic": traffic, "traffic_source": traffic_source,
+                     "traffic_stale": traffic_stale,
                      "algorithmic_bytes": {"forward": fwd_b, "backward": bwd_b},
                      "ms": {"forward": fwd_ms, "backward": bwd_ms},
                      "fwd_bwd_frac": (fwd_b + bwd_b) / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,

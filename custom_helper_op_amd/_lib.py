@@ -15,6 +15,7 @@ _DIMS = [_i64] * 8  # B,H,W,C,D,N,srcH,srcW
 #: name -> argument types, in the order of include/chop_costvol.h
 SIGNATURES = {
     "chop_abi_version": [],
+    "chop_init": [],
     "chop_last_error_string": [],
     "chop_set_kernel_family": [_int],
     "chop_last_kernel_family": [],

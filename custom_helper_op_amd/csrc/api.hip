@@ -327,6 +327,14 @@ void *scratch_on_current_device(hipError_t *err) {
   return p;
 }
 
+// The address if this device's look-up has been made, else nullptr.  No runtime call besides
+// hipGetDevice.
+void *scratch_if_known() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  return g_scratch_ptr[dev].load(std::memory_order_acquire);
+}
+
 }  // namespace
 }  // namespace chop
 
@@ -335,6 +343,16 @@ using namespace chop;
 extern "C" {
 
 int chop_abi_version(void) { return 1; }
+
+int chop_init(void) {
+  hipError_t err = hipSuccess;
+  if (scratch_on_current_device(&err) == nullptr) {
+    if (err == hipErrorNoDevice || err == hipErrorInvalidDevice)
+      return fail(CHOP_ERR_NO_DEVICE, std::string("chop_init: ") + hipGetErrorString(err));
+    return launch_status(err, "address of the built-in scratch");
+  }
+  return CHOP_OK;
+}
 
 const char *chop_last_error_string(void) { return g_last_error.c_str(); }
 
@@ -666,8 +684,20 @@ int chop_cost_volume_bwd_16_static(void *stream, int storage, int reduce, int ha
     return fail(CHOP_ERR_WORKSPACE, buf);
   }
   hipError_t err = hipSuccess;
-  void *ws = scratch_on_current_device(&err);
-  if (ws == nullptr) return launch_status(err, "address of the built-in scratch");
+  void *ws = scratch_if_known();
+  if (ws == nullptr) {
+    // first use on this device.  The look-up is a runtime query, not stream work: it does
+    // not belong inside a capture, so a capturing caller has to have made it before
+    // (chop_init, or any earlier call of this entry point on the device).
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cap) == hipSuccess &&
+        cap != hipStreamCaptureStatusNone)
+      return fail(CHOP_ERR_WORKSPACE,
+                  "the built-in scratch has not been located on this device yet: call "
+                  "chop_init() once per device before capturing");
+    ws = scratch_on_current_device(&err);
+    if (ws == nullptr) return launch_status(err, "address of the built-in scratch");
+  }
   // (the launch clears the part of the scratch it accumulates into: launch_tiled_backward /
   // launch_general_backward zero-fill both gradient images with a kernel before they add)
   return chop_cost_volume_bwd_16(stream, storage, reduce, half_centor, B, H, W, C, D, N, srcH,

@@ -273,6 +273,7 @@ hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream) {
 }
 
 hipError_t ZeroRanges::launch(hipStream_t stream) const {
+  if (bad) return hipErrorInvalidValue;
   if (count == 0) return hipSuccess;
   size_t most = 0;
   for (int i = 0; i < count; ++i) most = bytes[i] > most ? bytes[i] : most;

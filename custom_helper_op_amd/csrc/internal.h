@@ -142,16 +142,22 @@ hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
 // Up to three ranges zeroed by ONE launch (a launch costs ~5 us, the ranges are small):
 // collect them with add(), then launch().
 struct ZeroRanges {
-  unsigned char *ptr[3] = {nullptr, nullptr, nullptr};
-  size_t bytes[3] = {0, 0, 0};
+  static constexpr int kMax = 3;
+  unsigned char *ptr[kMax] = {nullptr, nullptr, nullptr};
+  size_t bytes[kMax] = {0, 0, 0};
   int count = 0;
+  bool bad = false;  // a range too many, or a NULL pointer with bytes: launch() reports it
   void add(void *p, size_t n) {
     if (n == 0) return;
+    if (count >= kMax || p == nullptr) {
+      bad = true;
+      return;
+    }
     ptr[count] = static_cast<unsigned char *>(p);
     bytes[count] = n;
     ++count;
   }
-  hipError_t launch(hipStream_t stream) const;
+  hipError_t launch(hipStream_t stream) const;  // hipErrorInvalidValue when `bad`
 };
 template <typename S>
 hipError_t launch_narrow(const float *from, S *to, int64_t count, hipStream_t stream);

@@ -53,6 +53,14 @@ enum { CHOP_REDUCE_MEAN = 0, CHOP_REDUCE_MIN = 1 };
 enum { CHOP_STORAGE_F16 = 1, CHOP_STORAGE_BF16 = 2 };
 
 int chop_abi_version(void);
+/* Optional set-up for the current device, outside any stream capture: locates the static
+ * scratch array of chop_cost_volume_bwd_16_static on this device (one runtime query, cached
+ * per device).  Every other entry point works without it; chop_cost_volume_bwd_16_static
+ * makes the same query on its first call on a device, unless that call is being captured
+ * into a HIP graph, in which case it returns CHOP_ERR_WORKSPACE and asks for this call.
+ * Returns CHOP_ERR_NO_DEVICE when there is no usable device.  No counterpart in the
+ * reference (its functors keep no state). */
+int chop_init(void);
 const char *chop_last_error_string(void);
 
 /* ---- CostVolume forward ------------------------------------------------------------
@@ -347,7 +355,8 @@ int chop_cost_volume_bwd_16(void *stream, int storage, int reduce, int half_cent
  * process ends; a shape whose chop_cost_volume_bwd16_workspace_bytes exceeds that is
  * rejected with CHOP_ERR_WORKSPACE.  The call allocates and frees nothing.  All calls on one
  * GPU share the array: calls that overlap in time on the same GPU (different streams or
- * host threads) race and must be serialised by the caller. */
+ * host threads) race and must be serialised by the caller.  A caller that captures the call
+ * into a HIP graph calls chop_init() (or this entry point) once on the device beforehand. */
 size_t chop_static_scratch_bytes(void);
 int chop_cost_volume_bwd_16_static(void *stream, int storage, int reduce, int half_centor,
                                    int64_t B, int64_t H, int64_t W, int64_t C, int64_t D,

@@ -555,13 +555,14 @@ def test_mvsnet_stage_full_size(oracle):
     _assert_family(0)
     assert cost.shape == (1, 128, 160, 192, 32)
     assert np.array_equal(host(mask), want_mask)
-    assert_forward_close(host(cost), want_cost)
+    # (how much of the comparison rests on the absolute floors: under one element in a hundred)
+    assert assert_forward_close(host(cost), want_cost, what="cost") < 0.01
     del cost
     want = oracle.cost_volume_bwd(*args, t["cost_grad"], want_mask, threads=16)
     got = chop.cost_volume_grad(*ins, dev(t["cost_grad"]), mask)
     _assert_family(0)
-    for g, w in zip(got, want):
-        assert_backward_close(host(g), w)
+    for g, w, name in zip(got, want, ("ref_grad", "src_grad", "base_plane_grad")):
+        assert assert_backward_close(host(g), w, what=name) < 0.01
 
 
 def test_large_batch_stress_full_size():
@@ -599,6 +600,14 @@ def test_large_batch_stress_full_size():
     del cost
     g1 = chop.cost_volume_grad(*ins, cg, mask)
     _assert_family(0)
+    # ref_grad and base_plane_grad are owned by their pixel: a band of them against the oracle
+    # run on that band alone (the first rows of a batch item, so no rows above it are needed)
+    b, r1 = 2, 16
+    want = oracle.cost_volume_bwd(t["ref"][b:b + 1, :r1], t["src"][b:b + 1], t["base_plane"][b:b + 1, :r1],
+                                  t["offsets"][b:b + 1], t["Rs"][b:b + 1], t["Ts"][b:b + 1],
+                                  host(cg[b:b + 1, :r1]), host(mask[b:b + 1, :r1]), threads=16)
+    assert_backward_close(host(g1[0][b:b + 1, :r1]), want[0], what="ref_grad band")
+    assert_backward_close(host(g1[2][b:b + 1, :r1]), want[2], what="base_plane_grad band")
     rg, sg = g1[0].double(), g1[1].double()
     assert abs(float(rg.sum() + sg.sum())) < 1e-4 * float(rg.abs().sum())
     cg.mul_(2.0)
@@ -606,6 +615,53 @@ def test_large_batch_stress_full_size():
     for a1, a2 in zip(g1, g2):
         scale = float(a1.abs().max())
         assert float((a2 - 2 * a1).abs().max()) <= 2e-4 * scale
+
+
+def test_volume_above_two_to_the_31_elements():
+    """The stress configuration with six batch items: 2.72 G cost elements (10.9 GB), so the
+    whole last batch item lies beyond element 2^31, where the reference switches to 64-bit
+    indices (cost_volume_kernels_gpu.cu.cc:313, :619).  The library's own choice of kernels
+    and the general kernels forced onto the same shape: mask bit-exact and cost within 1e-5
+    on a band of the last batch item, whole-volume properties, and for the backward
+    conservation plus the pixel-owned gradients of the band against the oracle."""
+    import oracle
+    wl = make_workload(5, with_cost_grad=False, batch=6)
+    t = wl.tensors
+    assert wl.B * wl.H * wl.W * wl.D * wl.C > 2 ** 31 + 2 ** 29
+    ins = _v1_inputs(t)
+    b, r1 = wl.B - 1, 16
+    assert b * wl.H * wl.W * wl.D * wl.C > 2 ** 31   # the band's rows start beyond 2^31
+    band = (t["ref"][b:b + 1, :r1], t["src"][b:b + 1], t["base_plane"][b:b + 1, :r1],
+            t["offsets"][b:b + 1], t["Rs"][b:b + 1], t["Ts"][b:b + 1])
+    want_cost, want_mask = oracle.cost_volume_fwd(*band, threads=16)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(31)
+    cg = torch.randn((wl.B, wl.H, wl.W, wl.D, wl.C), device="cuda", generator=gen)
+    want = oracle.cost_volume_bwd(*band, host(cg[b:b + 1, :r1]), want_mask, threads=16)
+    for family in (0, 1):
+        print("[case] above 2^31 elements, kernel family %d" % family, flush=True)
+        _lib.load().chop_set_kernel_family(family)
+        cost, mask = chop.cost_volume_raw(*ins)
+        _assert_family(family)
+        assert cost.numel() == 2717908992
+        assert np.array_equal(host(mask[b, :r1]), want_mask[0])
+        if family == 1:
+            assert np.array_equal(host(cost[b, :r1]), want_cost[0])   # literal operand order
+        else:
+            assert_forward_close(host(cost[b, :r1]), want_cost[0])
+        assert int(mask.min()) >= 0 and int(mask.max()) <= wl.N
+        assert float(cost.min()) >= 0.0
+        assert float((cost[b].abs() * (mask[b] == 0)).max()) == 0.0
+        del cost
+        g = chop.cost_volume_grad(*ins, cg, mask)
+        _assert_family(family)
+        rg, sg = g[0].double(), g[1].double()
+        assert abs(float(rg.sum() + sg.sum())) < 1e-4 * float(rg.abs().sum())
+        assert float(sg[b].abs().sum()) > 0.0
+        assert_backward_close(host(g[0][b:b + 1, :r1]), want[0], what="ref_grad band")
+        assert_backward_close(host(g[2][b:b + 1, :r1]), want[2], what="base_plane_grad band")
+        del g, rg, sg, mask
+        torch.cuda.empty_cache()
 
 
 # ---- five views: the six-view instantiation with one view missing ----------------------------

@@ -88,3 +88,56 @@ def test_static_scratch_entry_rejects_oversized_shapes():
                                             W, C, D, N, H, W, p, p, p, p, None, p, p, p, p, p, p, p)
     assert rc == 6  # CHOP_ERR_WORKSPACE
     assert b"built-in scratch" in lib.chop_last_error_string()
+
+
+def test_static_scratch_entry_in_a_captured_graph(oracle):
+    """The entry point captured into a HIP graph (chop_init() made the one runtime query
+    beforehand) and replayed on changed inputs, with eager work and synchronisations
+    between the replays: every replay against the oracle for the inputs of that replay."""
+    lib = _lib.load()
+    lib.chop_set_kernel_family(0)
+    _lib.check(lib.chop_init())
+    storage = "f16"
+    td = TORCH_DTYPE[storage]
+    wl = make_workload(3, hw=(24, 40))
+    t = wl.tensors
+    rng = np.random.default_rng(7)
+    ref, src = quantise(t["ref"], storage), quantise(t["src"], storage)
+    _, want_mask = oracle.cost_volume_fwd(ref, src, t["base_plane"], t["offsets"], t["Rs"], t["Ts"],
+                                          threads=8)
+    d_ref, d_src = dev(ref, td), dev(src, td)
+    d_cg = dev(quantise(t["cost_grad"], storage), td)
+    d_bp, d_off, d_rs, d_ts = (dev(t[k]) for k in ("base_plane", "offsets", "Rs", "Ts"))
+    d_mask = dev(want_mask)
+    rg, sg, bg = torch.empty_like(d_ref), torch.empty_like(d_src), torch.empty_like(d_bp)
+    dims = (wl.B, wl.H, wl.W, wl.C, wl.D, wl.N, wl.H, wl.W)
+
+    def call(stream):
+        return lib.chop_cost_volume_bwd_16_static(
+            stream, _STORAGE[storage], 0, 1, *dims, _ptr(d_ref), _ptr(d_src), _ptr(d_bp),
+            _ptr(d_off), None, _ptr(d_rs), _ptr(d_ts), _ptr(d_cg), _ptr(d_mask), _ptr(rg),
+            _ptr(sg), _ptr(bg))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _lib.check(call(side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        _lib.check(call(torch.cuda.current_stream().cuda_stream))
+    for replay in range(3):
+        print("\n[case] captured static-scratch backward, replay %d" % replay, flush=True)
+        new_ref = quantise(rng.standard_normal(ref.shape).astype(np.float32), storage)
+        new_cg = quantise(rng.standard_normal(t["cost_grad"].shape).astype(np.float32), storage)
+        d_ref.copy_(dev(new_ref, td))
+        d_cg.copy_(dev(new_cg, td))
+        rg.fill_(7.0), sg.fill_(-3.0), bg.fill_(11.0)   # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = oracle.cost_volume_bwd(new_ref, src, t["base_plane"], t["offsets"], t["Rs"], t["Ts"],
+                                      new_cg, want_mask)
+        for got, w in zip((rg, sg, bg), want):
+            np.testing.assert_allclose(host(got), w, rtol=1e-2, atol=1e-2 * max(rms(w), 1e-30))
