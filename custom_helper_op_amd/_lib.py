@@ -19,6 +19,7 @@ SIGNATURES = {
     "chop_last_error_string": [],
     "chop_set_kernel_family": [_int],
     "chop_last_kernel_family": [],
+    "chop_last_views_per_workgroup": [],
     "chop_cost_volume_bwd16_workspace_bytes": [_i64] * 7,
 }
 for _t in ("f32", "f64"):

@@ -17,6 +17,7 @@ namespace {
 thread_local std::string g_last_error = "";
 thread_local int g_kernel_family = 0;
 thread_local int g_last_family = 0;
+thread_local int g_last_views_per_workgroup = 0;
 
 int fail(int code, const std::string &msg) {
   g_last_error = msg;
@@ -336,6 +337,9 @@ void *scratch_if_known() {
 }
 
 }  // namespace
+
+void note_views_per_workgroup(int views) { g_last_views_per_workgroup = views; }
+
 }  // namespace chop
 
 using namespace chop;
@@ -343,6 +347,8 @@ using namespace chop;
 extern "C" {
 
 int chop_abi_version(void) { return 1; }
+
+int chop_last_views_per_workgroup(void) { return g_last_family == 2 ? g_last_views_per_workgroup : 0; }
 
 int chop_init(void) {
   hipError_t err = hipSuccess;

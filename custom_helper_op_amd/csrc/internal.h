@@ -137,6 +137,10 @@ hipError_t launch_tiled_forward_wide(const Args<S> &a, hipStream_t stream);
 template <typename S>
 hipError_t launch_tiled_backward_wide(const Args<S> &a, hipStream_t stream);
 
+// The tiled backward launcher reports how many views a workgroup took in turn (api.hip keeps
+// it per host thread for chop_last_views_per_workgroup).
+void note_views_per_workgroup(int views);
+
 // Utility launches.
 hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);
 // Up to three ranges zeroed by ONE launch (a launch costs ~5 us, the ranges are small):

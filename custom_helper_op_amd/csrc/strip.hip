@@ -22,7 +22,11 @@
 // are merged in registers and leave as one atomic add per tap and channel when the cell
 // changes (the reference issues one per voxel) -- a run that is still open at the end of a
 // chunk waits in LDS for the view's turn in the next chunk; the per-voxel depth gradient is
-// summed over the pixel's lanes in registers and stored once.
+// summed over the pixel's lanes in registers and stored once.  Wide pixels (16 lanes or more:
+// at most four pixels per wave, whose atomics would each carry one pixel's channels) put a
+// small write-back cache of texels in LDS between the runs and memory: consecutive runs of a
+// pixel and its neighbours hit the same texels, and a texel leaves as one atomic per channel
+// when another texel needs its slot.
 #include <type_traits>
 
 #include "internal.h"
@@ -38,6 +42,7 @@ struct StripGeom {
   int nseg, seg;        // depth segments, depths per segment (a multiple of kDB)
   int vg;               // views reprojected together: min(N, max(1, LPP / kDB))
   int carry;            // backward: open runs survive the end of a chunk (in LDS)
+  int cache;            // backward: a texel cache in LDS between the runs and memory
   int64_t tiles;        // ceil(B*H*W / PPW)
 };
 
@@ -85,6 +90,7 @@ template <typename R>
 struct StripRecords {
   R *f;      // NF fields of vg*PPW*kDB values each
   int *off;  // tap offset inside the view, -1: nothing to do
+  int *key;  // backward: the cell as (row << 16) | column
   int stride;
   __device__ __forceinline__ R &at(int field, int idx) { return f[field * stride + idx]; }
 };
@@ -95,13 +101,33 @@ __device__ __forceinline__ StripRecords<R> strip_records(unsigned char *smem, in
   r.stride = records;
   r.f = reinterpret_cast<R *>(smem);
   r.off = reinterpret_cast<int *>(smem + (size_t)NF * r.stride * sizeof(R));
+  r.key = r.off + records;
   return r;
 }
 
 // `records` = vg * PPW * (depths per chunk), then 64 values of staging
 template <typename R>
-constexpr size_t strip_lds_bytes(int nf, int records) {
-  return (size_t)records * (nf * sizeof(R) + sizeof(int)) + 64 * sizeof(R);
+constexpr size_t strip_lds_bytes(int nf, int records, int nints = 1) {
+  return (size_t)records * (nf * sizeof(R) + nints * sizeof(int)) + 64 * sizeof(R);
+}
+
+// Runs that are open at the end of a chunk: per view and lane four tap sums, the tap offset
+// and the cell.
+template <typename S>
+constexpr size_t strip_run_bytes(int64_t N) {
+  return (size_t)N * 64 * (4 * sizeof(typename Storage<S>::Real) + 2 * sizeof(int));
+}
+
+// Texel cache of the backward kernel: per view kCacheRows x kCacheCols slots addressed by the
+// low bits of the texel coordinates (direct-mapped), one value per lane of a pixel and a tag
+// (the texel's index over all images of the call, -1: empty) per slot.  Two rows by four
+// columns hold what a pixel and its neighbours in the strip work on at any time: the cells
+// of consecutive runs share two of their four texels, and a slot is needed again only two
+// rows or four columns further along the walk.
+constexpr int kCacheRows = 2, kCacheCols = 4, kCacheSlots = kCacheRows * kCacheCols;
+template <typename R>
+constexpr size_t strip_cache_bytes(int64_t N, int lpp) {
+  return (size_t)N * kCacheSlots * ((size_t)lpp * sizeof(R) + sizeof(int));
 }
 
 // ------------------------------------------------------------------------------------------
@@ -335,11 +361,21 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   StripRecords<R> rec = strip_records<R, 9>(smem, ppw * g.vg * kDB);
   // open runs between two chunks: per view the cell and its four tap sums, one slot per lane
   // (a lane only ever reads its own slots back)
-  R *s_run = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(9, ppw * g.vg * kDB));
+  R *s_run = reinterpret_cast<R *>(smem + strip_lds_bytes<R>(9, ppw * g.vg * kDB, 2));
   int *s_cur = reinterpret_cast<int *>(s_run + (size_t)N * 4 * 64);
   const bool carry = g.carry != 0;
   if (carry)
     for (int n = 0; n < N; ++n) s_cur[n * 64 + lane] = -1;
+  int *s_ckey = s_cur + (size_t)N * 64;  // the carried runs' cells as (row << 16) | column
+  // texel cache: values [view][slot][lane of the pixel], then the tags
+  const bool cache = g.cache != 0;
+  R *s_val = reinterpret_cast<R *>(reinterpret_cast<unsigned char *>(s_run) +
+                                   (carry ? strip_run_bytes<S>(N) : 0));
+  int *s_tag = reinterpret_cast<int *>(s_val + (size_t)N * kCacheSlots * lpp);
+  if (cache)
+    for (int k = lane; k < N * kCacheSlots; k += 64) s_tag[k] = -1;
+  const unsigned long long pix_lanes = lpp == 64 ? ~0ull : ((1ull << lpp) - 1ull);
+  const int64_t img_texels = (int64_t)srcH * srcW;
   R racc = R(0), dpart = R(0);
 
   for (int d0 = d_lo; d0 < d_hi; d0 += kDB) {
@@ -381,6 +417,7 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
           }
         }
         rec.off[ridx + j] = off;
+        rec.key[ridx + j] = off >= 0 ? ((s.fh << 16) | s.fw) : 0;
         rec.at(0, ridx + j) = s.k00;
         rec.at(1, ridx + j) = s.k01;
         rec.at(2, ridx + j) = s.k11;
@@ -399,22 +436,69 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         const S *view = a.src + view_off;
         Acc *gview = src_grad + view_off;
         int cur = -1, have = -1;  // cell of the open run, cell whose taps are in registers
+        int ckey = 0;             // the open run's cell as (row << 16) | column (cache only)
         R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
         R g00 = R(0), g01 = R(0), g11 = R(0), g10 = R(0);
         if (carry) {
           cur = s_cur[n * 64 + lane];
+          ckey = s_ckey[n * 64 + lane];
           g00 = s_run[(n * 4 + 0) * 64 + lane], g01 = s_run[(n * 4 + 1) * 64 + lane];
           g11 = s_run[(n * 4 + 2) * 64 + lane], g10 = s_run[(n * 4 + 3) * 64 + lane];
         }
-        auto flush = [&]() {
-          if (cur >= 0 && ch_ok) {
-            Acc *q = gview + cur;
-            if (g00 != R(0)) atomic_add(q, (Acc)g00);
-            if (g01 != R(0)) atomic_add(q + C, (Acc)g01);
-            if (g11 != R(0)) atomic_add(q + C + row_step, (Acc)g11);
-            if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
+        // The four texels of a finished run into the cache; called by all lanes of ONE pixel
+        // (the tag tests are uniform among them).  The four slots of a cell are distinct; their
+        // tags and values are read together, a miss writes the slot's old texel out first.
+        const int img0 = (int)(((int64_t)px.b * N + n) * img_texels);  // first texel of this view's image
+        auto cache_add_cell = [&]() {
+          const int fh = ckey >> 16, fw = ckey & 0xffff;
+          const int r0 = n * kCacheSlots + (fh & (kCacheRows - 1)) * kCacheCols;
+          const int r1 = n * kCacheSlots + ((fh + 1) & (kCacheRows - 1)) * kCacheCols;
+          const int c0 = fw & (kCacheCols - 1), c1 = (fw + 1) & (kCacheCols - 1);
+          const int slot[4] = {r0 + c0, r0 + c1, r1 + c1, r1 + c0};
+          const int t0 = img0 + fh * srcW + fw;
+          const int texel[4] = {t0, t0 + 1, t0 + srcW + 1, t0 + srcW};
+          const R add[4] = {g00, g01, g11, g10};
+          int tag[4];
+          R val[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) tag[k] = s_tag[slot[k]];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) val[k] = s_val[(size_t)slot[k] * lpp + cl];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (tag[k] == texel[k]) {
+              val[k] += add[k];
+            } else {
+              if (tag[k] >= 0 && val[k] != R(0) && cl < C)
+                atomic_add(src_grad + (int64_t)tag[k] * C + cl, (Acc)val[k]);
+              val[k] = add[k];
+              s_tag[slot[k]] = texel[k];
+            }
+            s_val[(size_t)slot[k] * lpp + cl] = val[k];
           }
-          g00 = g01 = g11 = g10 = R(0);
+        };
+        // The lanes with `fire` (whole pixels) hand over the tap sums of their run and clear
+        // them: straight to memory, or pixel by pixel into the cache (pixels of a strip hit
+        // the same texels, so they must not update a slot at the same time).
+        auto emit = [&](bool fire) {
+          if (!cache) {
+            if (fire && ch_ok) {
+              Acc *q = gview + cur;
+              if (g00 != R(0)) atomic_add(q, (Acc)g00);
+              if (g01 != R(0)) atomic_add(q + C, (Acc)g01);
+              if (g11 != R(0)) atomic_add(q + C + row_step, (Acc)g11);
+              if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
+            }
+          } else {
+            unsigned long long m = __ballot(fire);
+            while (m) {
+              const int lp = (__ffsll((long long)m) - 1) >> g.lpp_shift;
+              m &= ~(pix_lanes << (lp << g.lpp_shift));
+              if (p == lp) cache_add_cell();
+              strip_sync();
+            }
+          }
+          g00 = g01 = g11 = g10 = R(0);  // (a lane that does not fire has no open run)
         };
 #pragma unroll
         for (int jj = 0; jj < kDB; ++jj) {
@@ -422,8 +506,9 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
           if (off < 0) continue;
           const int64_t i = px.pix * D + d0 + jj;
           if (off != cur) {
-            flush();
+            emit(cur >= 0);
             cur = off;
+            ckey = rec.key[ridx + jj];
           }
           if (off != have) {
             have = off;
@@ -470,10 +555,11 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         }
         if (carry) {
           s_cur[n * 64 + lane] = cur;
+          s_ckey[n * 64 + lane] = ckey;
           s_run[(n * 4 + 0) * 64 + lane] = g00, s_run[(n * 4 + 1) * 64 + lane] = g01;
           s_run[(n * 4 + 2) * 64 + lane] = g11, s_run[(n * 4 + 3) * 64 + lane] = g10;
         } else {
-          flush();
+          emit(cur >= 0);
         }
       }
     }  // group of views
@@ -501,6 +587,20 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
       if (g10 != R(0)) atomic_add(q + row_step, (Acc)g10);
     }
   }
+  if (cache) {
+    // everything the cache still holds
+    strip_sync();
+    for (int s0 = 0; s0 < N * kCacheSlots; s0 += ppw) {
+      const int slot = s0 + p;
+      if (slot < N * kCacheSlots && cl < C) {
+        const int tag = s_tag[slot];
+        if (tag >= 0) {
+          const R v = s_val[(size_t)slot * lpp + cl];
+          if (v != R(0)) atomic_add(src_grad + (int64_t)tag * C + cl, (Acc)v);
+        }
+      }
+    }
+  }
   if (ch_ok && !FEAT) {
     Acc *q = ref_grad + px.pix * C + cl;
     if (g.nseg == 1)
@@ -519,10 +619,7 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   }
 }
 
-template <typename S>
-constexpr size_t strip_run_bytes(int64_t N) {
-  return (size_t)N * 64 * (4 * sizeof(typename Storage<S>::Real) + sizeof(int));
-}
+
 
 template <typename S>
 StripGeom strip_geometry(const Args<S> &a) {
@@ -541,6 +638,12 @@ StripGeom strip_geometry(const Args<S> &a) {
   g.nseg = (int)((a.D + g.seg - 1) / g.seg);
   // carried runs: N * 64 lanes * (4 sums + cell); given up beyond 16 KiB
   g.carry = strip_run_bytes<S>(a.N) <= 16384;
+  // Wide pixels: the texel cache between the runs and memory, as long as
+  // it stays small (8 KiB: four views of 32 double-precision lanes) and a texel's index over
+  // all images of the call fits its 32-bit tag.
+  using R = typename Storage<S>::Real;
+  g.cache = lpp >= 16 && strip_cache_bytes<R>(a.N, lpp) <= 8192 &&
+            a.B * a.N * a.srcH * a.srcW < (int64_t)1 << 31 && a.srcH < 32768 && a.srcW < 65536;
   return g;
 }
 
@@ -608,8 +711,9 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
       zero.add(a.depth_grad, (size_t)a.pixels() * sizeof(R));
   }
   if ((err = zero.launch(stream)) != hipSuccess) return err;
-  const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB) +
-                      (g.carry ? strip_run_bytes<S>(a.N) : 0);
+  const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB, 2) +
+                      (g.carry ? strip_run_bytes<S>(a.N) : 0) +
+                      (g.cache ? strip_cache_bytes<R>(a.N, 1 << g.lpp_shift) : 0);
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
   if (a.corr == WARP_ONLY) {
     strip_backward_kernel<S, 4, 0><<<grid, block, smem, stream>>>(a, g);

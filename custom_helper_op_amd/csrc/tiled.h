@@ -156,6 +156,39 @@ __device__ __forceinline__ void store_vec(S *p, const float *in) {
     *q = v;
 }
 
+// The same load without the conversion: CNT elements as they lie in memory, in 32-bit words
+// (a single 16-bit element in the low half of one word).  A wave that widens 16-bit values
+// right after the load waits for memory at that point; keeping the words and widening them
+// where they are used lets the wait fall behind whatever work sits in between.
+template <typename S, int CNT>
+constexpr int raw_words() { return (CNT * (int)sizeof(S) + 3) / 4; }
+template <typename S, int CNT, bool STREAM>
+__device__ __forceinline__ void load_raw(const S *p, uint32_t *out) {
+  constexpr int BYTES = CNT * (int)sizeof(S);
+  using RawT = typename Raw<BYTES>::type;
+  const RawT *q = reinterpret_cast<const RawT *>(p);
+  const RawT v = STREAM ? __builtin_nontemporal_load(q) : *q;
+  if constexpr (BYTES <= 4) {
+    out[0] = (uint32_t)v;
+  } else {
+#pragma unroll
+    for (int k = 0; k < BYTES / 4; ++k) out[k] = v[k];
+  }
+}
+template <typename S, int CNT>
+__device__ __forceinline__ void widen_raw(const uint32_t *in, float *out) {
+  constexpr int BYTES = CNT * (int)sizeof(S);
+  constexpr int PER_WORD = 4 / (int)sizeof(S);
+  if constexpr (BYTES == 2) {
+    float two[2];
+    widen_word<S>(in[0], two);
+    out[0] = two[0];
+  } else {
+#pragma unroll
+    for (int k = 0; k < BYTES / 4; ++k) widen_word<S>(in[k], out + k * PER_WORD);
+  }
+}
+
 // Orders this wave's LDS traffic: the lanes of a wavefront execute in lockstep and the
 // LDS returns a wave's operations in issue order, so only the compiler has to be kept
 // from moving accesses across the phase boundary.
@@ -1224,30 +1257,65 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
   ox = nx;
 }
 
-// Writes out everything a window holds, at the end of the workgroup: all LDS reads are issued
-// together (the registers of the main loop are free by then), then all the atomics, so the
-// wave waits for the LDS once instead of once per group of texels.
+// Bitwise OR over the 64 lanes, in registers (as wave_min).
+__device__ __forceinline__ unsigned wave_or(unsigned v) {
+  v |= (unsigned)__builtin_amdgcn_update_dpp((int)v, (int)v, 0xB1, 0xf, 0xf, false);
+  v |= (unsigned)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x4E, 0xf, 0xf, false);
+  v |= (unsigned)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x141, 0xf, 0xf, false);
+  v |= (unsigned)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x140, 0xf, 0xf, false);
+  return (unsigned)__builtin_amdgcn_readlane((int)v, 0) | (unsigned)__builtin_amdgcn_readlane((int)v, 16) |
+         (unsigned)__builtin_amdgcn_readlane((int)v, 32) | (unsigned)__builtin_amdgcn_readlane((int)v, 48);
+}
+
+// Writes out everything a window holds, when its view is done: row by row of the ring
+// buffer, and only the rows some accepted cell of this view ever mapped to (`rows`: bit r
+// set when a cell used ring row r; a short sweep over few hypotheses touches three or four
+// of the eight, and the untouched ones need neither their LDS reads nor their address
+// arithmetic).  All LDS reads of a row are issued together, then its atomics.
 template <int VEC, int LPP>
 __device__ __forceinline__ void window_flush_all(int oy, int ox, const float *data, float *gview,
-                                                 int srcW, int lane) {
+                                                 int srcW, int lane, unsigned rows) {
   using WN = Window<VEC, LPP>;
   if (oy == WN::kNone) return;
   wave_sync();  // the last adds are complete and visible
   constexpr int C = WN::C;
-  constexpr int NI = WN::SLOTS * C / 64;  // instructions of 64 consecutive floats
-  constexpr int BATCH = NI < 32 ? NI : 32;
-  static_assert(NI % BATCH == 0, "whole batches");
+  constexpr int PER_ROW = WN::COLS * C / 64;  // instructions of 64 consecutive floats per row
+  static_assert(WN::COLS * C % 64 == 0, "whole instructions per window row");
+  if (__popc(rows) > WN::ROWS * 5 / 8) {
+    // (nearly) every row in use, as after a long sweep: the whole window in batches of 32
+    // instructions whose LDS reads go out together, so that the wave waits for the LDS once
+    // per batch instead of once per row (315 against 325 us on the MVSNet-stage workload)
+    constexpr int NI = WN::SLOTS * C / 64;
+    constexpr int BATCH = NI < 32 ? NI : 32;
+    static_assert(NI % BATCH == 0, "whole batches");
 #pragma unroll 1
-  for (int i0 = 0; i0 < NI; i0 += BATCH) {
-    float v[BATCH];
+    for (int i0 = 0; i0 < NI; i0 += BATCH) {
+      float v[BATCH];
 #pragma unroll
-    for (int u = 0; u < BATCH; ++u) v[u] = data[(i0 + u) * 64 + lane];
+      for (int u = 0; u < BATCH; ++u) v[u] = data[(i0 + u) * 64 + lane];
 #pragma unroll
-    for (int u = 0; u < BATCH; ++u) {
-      const int e = (i0 + u) * 64 + lane;  // float index inside the window
-      const int s = e / C, ch = e - s * C;
-      const int ry = s / WN::COLS, rx = s - ry * WN::COLS;
-      const int y = oy + ((ry - oy) & (WN::ROWS - 1)), x = ox + ((rx - ox) & (WN::COLS - 1));
+      for (int u = 0; u < BATCH; ++u) {
+        const int e = (i0 + u) * 64 + lane;  // float index inside the window
+        const int sl = e / C, ch = e - sl * C;
+        const int ry = sl / WN::COLS, rx = sl - ry * WN::COLS;
+        const int y = oy + ((ry - oy) & (WN::ROWS - 1)), x = ox + ((rx - ox) & (WN::COLS - 1));
+        if (v[u] != 0.f) atomic_add(gview + ((int64_t)(y * srcW + x) * C + ch), v[u]);
+      }
+    }
+    return;
+  }
+#pragma unroll 1
+  for (int ry = 0; ry < WN::ROWS; ++ry) {
+    if (!((rows >> ry) & 1u)) continue;  // uniform
+    const int y = oy + ((ry - oy) & (WN::ROWS - 1));
+    float v[PER_ROW];
+#pragma unroll
+    for (int u = 0; u < PER_ROW; ++u) v[u] = data[(ry * PER_ROW + u) * 64 + lane];
+#pragma unroll
+    for (int u = 0; u < PER_ROW; ++u) {
+      const int e = u * 64 + lane;  // float index inside the row
+      const int rx = e / C, ch = e - rx * C;
+      const int x = ox + ((rx - ox) & (WN::COLS - 1));
       // (a slot that was never added to holds zero: texels outside the image never are)
       if (v[u] != 0.f) atomic_add(gview + ((int64_t)(y * srcW + x) * C + ch), v[u]);
     }
@@ -1419,8 +1487,11 @@ constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 :
 // PV: the depth hypotheses come from a per-voxel depth_grid (and the depth gradient is per
 // voxel); a compile-time flag, because the kernel without the unused variant's code is
 // measurably faster than one that tests a.depth_grid at run time.
+// VLOOP: the workgroup's view group holds several views, which take turns (g.vper of them).
+// A compile-time flag: the loop around the kernel's body costs the wide instantiations
+// registers they do not have (the 32-channel kernel spills with it).
 template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true,
-          bool PV = (CORR == 1)>
+          bool PV = (CORR == 1), bool VLOOP = false>
 __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
   using WN = Window<VEC, LPP>;
@@ -1447,12 +1518,6 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   // CORR 3 only: reference rows, sample rows
   float *s_v3 = s_stage + 4 * WN::C + (LPP <= kClaimLanes ? WN::SLOTS : 0);
   static_assert(CORR != 3 || (NV == 1 && LPP > 1 && VEC == 4), "CostVolumeV3: one view, wide pixels");
-  for (int k = t.lane * 4; k < NV * WN::SLOTS * WN::STRIDE; k += 256)
-    *reinterpret_cast<float4 *>(s_data + k) = make_float4(0.f, 0.f, 0.f, 0.f);
-
-  Cameras<NV> cam;
-  load_cameras<S, NV>(a, t.b, t.view0, static_cast<float>(t.w) + half,
-                      static_cast<float>(t.h) + half, cam);
   const float base = per_voxel_depth ? 0.f : a.base_plane[t.pix];
   float ref[VEC];
   if constexpr (CORR != 4) {
@@ -1468,36 +1533,12 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   }
   const int64_t view_elems = (int64_t)srcH * srcW * C;
   float *src_grad_img = kWide ? a.src_grad_acc : reinterpret_cast<float *>(a.src_grad);
-  const S *view[NV];
-  float *gview[NV];  // gradient image of the view, no lane offset
-  int oy[NV], ox[NV];
-#pragma unroll
-  for (int n = 0; n < NV; ++n) {
-    const int64_t vo = ((int64_t)t.b * N + (t.view0 + n < N ? t.view0 + n : 0)) * view_elems;
-    view[n] = a.src + vo;  // uniform: taps are addressed as base + 32-bit lane offset
-    gview[n] = src_grad_img + vo;
-    oy[n] = ox[n] = WN::kNone;
-  }
   const int row_step = srcW * C;
   const unsigned lane_ch = (unsigned)(t.cl * VEC);
-
-  float tap[NV][4][VEC], sg[NV][4][VEC];
-  int cur[NV];     // tap offset of the open run, -1: none
-  int2 cell[NV];   // its slots and key (bit 31: inside the window)
-#pragma unroll
-  for (int n = 0; n < NV; ++n) {
-    cur[n] = -1;
-    cell[n] = make_int2(0, 0);
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-#pragma unroll
-      for (int c = 0; c < VEC; ++c) sg[n][k][c] = 0.f;
-  }
   float racc[VEC];
 #pragma unroll
   for (int c = 0; c < VEC; ++c) racc[c] = 0.f;
   float dacc = 0.f;  // base-plane gradient partial of this lane
-  wave_sync();
 
   // CORR: 0 squared difference per channel, 1 group correlation, 2 squared difference
   // summed over all channels (one upstream gradient per voxel), 4 the warp alone: one
@@ -1518,13 +1559,54 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
   // element steps from one depth to the next in the upstream gradient and in the mask
   const int cg_step = CORR == 4 ? N * C : OC;
   const int cnt_step = CORR == 4 ? N : mask_w;
+  const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
+  // The views of this workgroup's group take turns (NV at a time; NV = 1 in every launch):
+  // each gets the scatter window to itself and leaves it empty.  What belongs to the pixel
+  // (reference gradient, depth gradients, the upstream rows in the caches) is shared, so a
+  // group of all N views needs no atomics for the pixel-owned outputs.
+  const int first_view = t.view0;
+  const int group_views = VLOOP ? min(g.vper > NV ? g.vper : NV, N - first_view) : NV;
+  for (int vi = 0; vi < group_views; vi += NV) {
+  t.view0 = first_view + vi;
+  for (int k = t.lane * 4; k < NV * WN::SLOTS * WN::STRIDE; k += 256)
+    *reinterpret_cast<float4 *>(s_data + k) = make_float4(0.f, 0.f, 0.f, 0.f);
+  Cameras<NV> cam;
+  load_cameras<S, NV>(a, t.b, t.view0, static_cast<float>(t.w) + half,
+                      static_cast<float>(t.h) + half, cam);
+  const S *view[NV];
+  float *gview[NV];  // gradient image of the view, no lane offset
+  int oy[NV], ox[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    const int64_t vo = ((int64_t)t.b * N + (t.view0 + n < N ? t.view0 + n : 0)) * view_elems;
+    view[n] = a.src + vo;  // uniform: taps are addressed as base + 32-bit lane offset
+    gview[n] = src_grad_img + vo;
+    oy[n] = ox[n] = WN::kNone;
+  }
+  float tap[NV][4][VEC], sg[NV][4][VEC];
+  int cur[NV];     // tap offset of the open run, -1: none
+  int2 cell[NV];   // its slots and key (bit 31: inside the window)
+  unsigned ring_rows[NV];  // ring rows of the window this lane's accepted cells mapped to
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    cur[n] = -1;
+    ring_rows[n] = 0u;
+    cell[n] = make_int2(0, 0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) sg[n][k][c] = 0.f;
+  }
   const S *cg_lane =
       CORR == 4 ? a.cost_grad + (t.pix * D * N + t.view0) * C + t.cl * VEC
                 : a.cost_grad + t.pix * D * OC + (kVoxelGrad ? 0 : t.cl * (CORR ? gv : VEC));
-  const float *dv_src = per_voxel_depth ? a.depth_grid + t.pix * D : a.offsets + (int64_t)t.b * D;
   const int32_t *cnt_src = CORR == 4 ? a.mask_in + t.pix * D * N + t.view0
                                      : a.mask_in + t.pix * D * mask_w;
   const int32_t *mask_lane = cnt_src + t.cl * (CORR ? gv : VEC);  // this lane's part of a mask row
+  // the pixel's depth gradients: the first view of a group that holds them all stores, the
+  // later ones add (same lane, same address); several groups add atomically
+  const bool dg_store = g.ngroups == 1 && vi == 0, dg_own = g.ngroups == 1;
+  wave_sync();
   for (int d0 = d_lo; d0 < d_hi; d0 += LPP) {
     // Depth hypothesis and valid-view count of lane (p, j)'s voxel: requested before the
     // chunk's upstream-gradient rows, because loads return in order and the reprojection
@@ -1561,17 +1643,32 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
     // two-view benchmark tensors and save 2 % with warm caches, but the rows they leave
     // behind in L2 and the memory-side cache cost the next forward launch 5 us, and after
     // other work has filled the caches with dirty lines they are 3 % slower than streaming.
-    float cgr[kVoxelGrad ? 1 : PF][VEC];
+    // (whole rows are kept as loaded and widened to float where a depth uses them; group
+    // rows, whose width is a run-time value, are widened here and kept as float bits)
+    uint32_t cgw[kVoxelGrad ? 1 : PF][(CORR == 0 || CORR == 4) ? raw_words<S, VEC>() : VEC];
     int mrow[kMaskRows ? PF : 1][VEC];
     auto load_rows = [&](int first) {
+      if constexpr (CORR == 1) {
+        // the group width is a run-time value: one branch around all of the chunk's loads, so
+        // that they go out together (a branch per row makes each row wait for the one before)
+        auto group_rows = [&](auto cnt) {
+          constexpr int CNT = decltype(cnt)::value;
+#pragma unroll
+          for (int jj = 0; jj < PF; ++jj) {
+            const int d = min(first + jj, d_hi - 1);
+            load_vec<S, CNT, true>(cg_lane + (int64_t)d * cg_step, reinterpret_cast<float *>(cgw[jj]));
+          }
+        };
+        if (g.sub == 1) group_rows(std::integral_constant<int, VEC>());
+        else if (g.sub == 2) group_rows(std::integral_constant<int, VEC / 2>());
+        else if (g.sub == 4) group_rows(std::integral_constant<int, VEC / 4>());
+        else if constexpr (VEC >= 8) group_rows(std::integral_constant<int, VEC / 8>());
+      }
 #pragma unroll
       for (int jj = 0; jj < PF; ++jj) {
         const int d = min(first + jj, d_hi - 1);
         const S *src_cg = cg_lane + (int64_t)d * cg_step;
-        if (CORR == 0 || CORR == 4)
-          load_vec<S, VEC, true>(src_cg, cgr[jj]);
-        else
-          load_groups<S, VEC, true>(src_cg, cgr[jj], g.sub);
+        if constexpr (CORR == 0 || CORR == 4) load_raw<S, VEC, true>(src_cg, cgw[jj]);
         if constexpr (kMaskRows) {
           const int32_t *m = mask_lane + (int64_t)d * OC;
           const int cntv = CORR == 0 ? VEC : gv;
@@ -1640,6 +1737,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
         // the last chunk.  Usually it already does (one vote); otherwise it is centred on
         // their bounding box, and whatever still sticks out is marked for the memory path.
         const bool valid = hit.off >= 0;
+        if (valid) {
+          const unsigned fh = (unsigned)hit.key >> 16;
+          ring_rows[n] |= (1u << (fh & (WN::ROWS - 1))) | (1u << ((fh + 1u) & (WN::ROWS - 1)));
+        }
         bool in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
         chunk_out[n] = false;
         if (__ballot(!(in_new && (cur[n] < 0 || cell[n].y < 0))) != 0ull) {
@@ -1756,7 +1857,14 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       if (NV == 1 ? rec_off[0] >= 0 : scl != 0.f) {
         float cg[VEC];
         {
-          const float *raw = cgr[kVoxelGrad ? 0 : jj % PF];
+          float raw[VEC];
+          if constexpr (!kVoxelGrad) {
+            if (CORR == 0 || CORR == 4)
+              widen_raw<S, VEC>(cgw[jj % PF], raw);
+            else
+#pragma unroll
+              for (int c = 0; c < VEC; ++c) raw[c] = __uint_as_float(cgw[jj % PF][c]);
+          }
           if constexpr (kVoxelGrad) {
 #pragma unroll
             for (int c = 0; c < VEC; ++c) cg[c] = scl;
@@ -1870,8 +1978,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
           if (t.cl == 0) lds_at<float>(smem, p4, kDst + (jj * PPW) * 4) = tot;
         } else {
           if (t.pix_ok) {
-            if (g.ngroups == 1)
+            if (dg_store)
               a.depth_grad[t.pix * D + d] = dvox;
+            else if (dg_own)
+              a.depth_grad[t.pix * D + d] += dvox;
             else
               atomic_add(a.depth_grad + t.pix * D + d, dvox);
           }
@@ -1885,10 +1995,13 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
       if (DG && per_voxel_depth) {
         const int d = d0 + t.cl;
         if (d < d_hi && t.pix_ok) {
-          if (g.ngroups == 1)
-            a.depth_grad[t.pix * D + d] = lds_at<float>(smem, q4, kDst);
+          const float tot = lds_at<float>(smem, q4, kDst);
+          if (dg_store)
+            a.depth_grad[t.pix * D + d] = tot;
+          else if (dg_own)
+            a.depth_grad[t.pix * D + d] += tot;
           else
-            atomic_add(a.depth_grad + t.pix * D + d, lds_at<float>(smem, q4, kDst));
+            atomic_add(a.depth_grad + t.pix * D + d, tot);
         }
         wave_sync();
       }
@@ -1910,7 +2023,9 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(c
 #pragma unroll
   for (int n = 0; n < NV; ++n)
     window_flush_all<VEC, LPP>(oy[n], ox[n], s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
-                               t.lane);
+                               t.lane, wave_or(ring_rows[n]));
+  wave_sync();  // the next view clears the window
+  }  // views of the group
 
   // pixel-owned gradients: one store when this workgroup saw every depth, otherwise one
   // atomic add per depth segment into the zero-filled outputs

@@ -415,6 +415,11 @@ int chop_set_kernel_family(int family);
 /* Which family served the last forward/backward call of this thread: 0 none yet,
  * 1 general kernels, 2 tiled kernels, 3 strip kernels. */
 int chop_last_kernel_family(void);
+/* How many source views one workgroup of the last tiled backward call of this thread went
+ * through in turn (1: every view had workgroups of its own; N: narrow pixels on a large
+ * image, all views of a pixel tile in one workgroup); 0 if the last backward call did not run
+ * the tiled kernels.  For the tests. */
+int chop_last_views_per_workgroup(void);
 
 #ifdef __cplusplus
 }
