@@ -52,6 +52,15 @@ __device__ __forceinline__ void strip_sync() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// 1 / x to within an ulp or two, for the backward's factors (a full IEEE division costs about
+// ten instructions in float and fifty in double; the gradients are compared at 1e-4).
+__device__ __forceinline__ float quick_recip(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double quick_recip(double x) {
+  double r = __builtin_amdgcn_rcp(x);
+  r = __builtin_fma(__builtin_fma(-x, r, 1.0), r, r);
+  return __builtin_fma(__builtin_fma(-x, r, 1.0), r, r);
+}
+
 // Sum over the 2^shift consecutive lanes of a pixel, left in every one of them.
 template <typename R>
 __device__ __forceinline__ R pixel_sum(R v, int shift) {
@@ -382,6 +391,20 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
     R dvox[kDB];
 #pragma unroll
     for (int jj = 0; jj < kDB; ++jj) dvox[jj] = R(0);
+    // This lane's upstream gradients (and, for the MIN reduce, winners) of the chunk's depths,
+    // requested together and ahead of the reprojection: fetched one by one where a depth
+    // uses them, every depth of every wave waits for memory (the kernel spent two thirds of
+    // its time in such waits).  They serve all views.
+    R cgv[kDB];
+    int win[REDUCE != 0 ? kDB : 1];
+    if constexpr (!FEAT) {
+#pragma unroll
+      for (int jj = 0; jj < kDB; ++jj) {
+        const int64_t i = px.pix * D + min(d0 + jj, d_hi - 1);
+        cgv[jj] = Storage<S>::load(a.cost_grad + i * OC + oc);
+        if constexpr (REDUCE != 0) win[jj] = a.mask_in[i * OC + oc];
+      }
+    }
     for (int n0 = 0; n0 < N; n0 += g.vg) {
       const int nv = min(g.vg, N - n0);
       strip_sync();
@@ -394,25 +417,33 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         Sample<R> s;
         s.k00 = s.k01 = s.k11 = s.k10 = s.dh = s.dw = R(0);
         R fh = R(0), fw = R(0), cnt = R(1);
+        // every load of this item goes out before the first test, so that the item waits for
+        // memory once (mask, then depth, then camera, each behind a branch, were three waits)
+        const int64_t i = px.pix * D + min(d, d_hi - 1);
+        // FeatureAggregate: 1 / 0 per (voxel, view), :261-263
+        const int32_t m0 = FEAT ? a.mask_in[i * N + n0 + nl] : a.mask_in[REDUCE == 0 ? i : i * OC];
+        const R dval = per_voxel ? a.depth_grid[i] : a.offsets[(int64_t)px.b * D + min(d, d_hi - 1)];
+        R Rm[9], Tv[3];
+#pragma unroll
+        for (int k = 0; k < 9; ++k) Rm[k] = a.Rs[cam * 9 + k];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) Tv[k] = a.Ts[cam * 3 + k];
         if (d < d_hi && px.ok) {
-          const int64_t i = px.pix * D + d;
-          // FeatureAggregate: 1 / 0 per (voxel, view), :261-263
-          const int32_t m0 = FEAT ? a.mask_in[i * N + n0 + nl] : a.mask_in[REDUCE == 0 ? i : i * OC];
           // MEAN skips a voxel no view reached (:367), MIN one whose first entry is negative (:484)
           if (REDUCE == 0 ? (m0 > 0) : (m0 >= 0)) {
-            const R depth = per_voxel ? a.depth_grid[i] : base + a.offsets[(int64_t)px.b * D + d];
-            project(a.Rs + cam * 9, a.Ts + cam * 3, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
+            const R depth = per_voxel ? dval : base + dval;
+            project(Rm, Tv, px.ref_w, px.ref_h, depth, a.half, srcH, srcW, s);
             if (s.state == 2) {
               off = (s.fh * srcW + s.fw) * C;
-              const R zz = s.z * s.z;
-              fh = (s.h_coef * s.z - s.z_coef * s.h3d) / zz;
-              fw = (s.w_coef * s.z - s.z_coef * s.w3d) / zz;
+              const R izz = quick_recip(s.z * s.z);
+              fh = (s.h_coef * s.z - s.z_coef * s.h3d) * izz;
+              fw = (s.w_coef * s.z - s.z_coef * s.w3d) * izz;
               if constexpr (FEAT)
                 cnt = R(1);
               else if constexpr (AGG)  // cost_aggregate_kernels_gpu.cu.cc:388, :502
-                cnt = R(1) / static_cast<R>(REDUCE == 0 ? (int64_t)m0 * C : (int64_t)C);
+                cnt = quick_recip(static_cast<R>(REDUCE == 0 ? (int64_t)m0 * C : (int64_t)C));
               else
-                cnt = R(1) / static_cast<R>(m0);
+                cnt = quick_recip(static_cast<R>(m0));
             }
           }
         }
@@ -435,6 +466,13 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         const int64_t view_off = ((int64_t)px.b * N + n) * srcH * srcW * C + (ch_ok ? cl : 0);
         const S *view = a.src + view_off;
         Acc *gview = src_grad + view_off;
+        if constexpr (FEAT) {  // an upstream row per view
+#pragma unroll
+          for (int jj = 0; jj < kDB; ++jj) {
+            const int64_t i = px.pix * D + min(d0 + jj, d_hi - 1);
+            cgv[jj] = Storage<S>::load(a.cost_grad + (i * N + n) * C + (ch_ok ? cl : 0));
+          }
+        }
         int cur = -1, have = -1;  // cell of the open run, cell whose taps are in registers
         int ckey = 0;             // the open run's cell as (row << 16) | column (cache only)
         R v00 = R(0), v01 = R(0), v11 = R(0), v10 = R(0);
@@ -504,7 +542,6 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         for (int jj = 0; jj < kDB; ++jj) {
           const int off = rec.off[ridx + jj];
           if (off < 0) continue;
-          const int64_t i = px.pix * D + d0 + jj;
           if (off != cur) {
             emit(cur >= 0);
             cur = off;
@@ -517,12 +554,12 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
             v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
           }
           if (!ch_ok) continue;
-          if (REDUCE != 0 && a.mask_in[i * OC + oc] != n) continue;  // another view won (:553)
+          if constexpr (REDUCE != 0)
+            if (win[jj] != n) continue;  // another view won (:553)
           const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
                   k10 = rec.at(3, ridx + jj);
           const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
-          const R cg = FEAT ? Storage<S>::load(a.cost_grad + (i * N + n) * C + cl)
-                            : Storage<S>::load(a.cost_grad + i * OC + oc);
+          const R cg = cgv[jj];
           // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
           // reference's division (one division per voxel in phase 1 instead of one per element)
           const R inv = rec.at(8, ridx + jj);
@@ -642,7 +679,9 @@ StripGeom strip_geometry(const Args<S> &a) {
   // it stays small (8 KiB: four views of 32 double-precision lanes) and a texel's index over
   // all images of the call fits its 32-bit tag.
   using R = typename Storage<S>::Real;
-  g.cache = lpp >= 16 && strip_cache_bytes<R>(a.N, lpp) <= 8192 &&
+  // (float64 only: its atomics move twice the bytes; with 32-bit elements the cache's own
+  // work costs more than it saves, 749 against 735 us at 24 channels)
+  g.cache = sizeof(R) == 8 && lpp >= 16 && strip_cache_bytes<R>(a.N, lpp) <= 8192 &&
             a.B * a.N * a.srcH * a.srcW < (int64_t)1 << 31 && a.srcH < 32768 && a.srcW < 65536;
   return g;
 }
