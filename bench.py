@@ -111,10 +111,10 @@ class Runner:
             rc = fn(s, self.red, 1, *self.dims, p(self.ref), p(self.src), p(self.base_plane),
                     p(self.offsets), p(self.Rs), p(self.Ts), p(self.cost), p(self.mask))
         elif self.v3:
-            rc = lib.chop_cost_volume_v3_fwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
-                                                 p(self.ref), p(self.src), p(self.base_plane),
-                                                 p(self.offsets), p(self.Rs), p(self.Ts),
-                                                 p(self.cost), p(self.mask))
+            fn = lib.chop_cost_volume_v3_fwd_f64 if self.f64 else lib.chop_cost_volume_v3_fwd_f32
+            rc = fn(s, self.red, 1, *self.dims, self.wl.groups, p(self.ref), p(self.src),
+                    p(self.base_plane), p(self.offsets), p(self.Rs), p(self.Ts), p(self.cost),
+                    p(self.mask))
         elif self.feat:
             fn = lib.chop_feature_aggregate_fwd_f64 if self.f64 else lib.chop_feature_aggregate_fwd_f32
             rc = fn(s, 1, *self.dims, p(self.src), p(self.base_plane), p(self.offsets), p(self.Rs),
@@ -154,9 +154,9 @@ class Runner:
             rc = fn(s, self.red, 1, *self.dims, p(self.ref), p(self.src), p(self.base_plane),
                     p(self.offsets), p(self.Rs), p(self.Ts), *tail)
         elif self.v3:
-            rc = lib.chop_cost_volume_v3_bwd_f32(s, self.red, 1, *self.dims, self.wl.groups,
-                                                 p(self.ref), p(self.src), p(self.base_plane),
-                                                 p(self.offsets), p(self.Rs), p(self.Ts), *tail)
+            fn = lib.chop_cost_volume_v3_bwd_f64 if self.f64 else lib.chop_cost_volume_v3_bwd_f32
+            rc = fn(s, self.red, 1, *self.dims, self.wl.groups, p(self.ref), p(self.src),
+                    p(self.base_plane), p(self.offsets), p(self.Rs), p(self.Ts), *tail)
         elif self.feat:
             fn = lib.chop_feature_aggregate_bwd_f64 if self.f64 else lib.chop_feature_aggregate_bwd_f32
             rc = fn(s, 1, *self.dims, p(self.src), p(self.base_plane), p(self.offsets), p(self.Rs),
@@ -368,9 +368,9 @@ def main():
     wl = make_workload(a.workload, with_cost_grad=False)
     wl.reduce_method = a.reduce
     if a.float64 or a.channels:
-        if wl.op != "v1" or wl.storage != "f32" or a.v3:
+        if wl.op != "v1" or wl.storage != "f32":
             sys.exit("bench.py: --float64 / --channels need a float32 CostVolume workload (1, 2 or 5), "
-                     "alone or with --aggregate / --feature")
+                     "alone or with --aggregate / --v3 / --feature")
         if a.channels:
             if not 1 <= a.channels <= wl.C:
                 sys.exit("bench.py: --channels must be 1..%d for this workload" % wl.C)
@@ -385,7 +385,7 @@ def main():
             sys.exit("bench.py: --aggregate needs a float32 CostVolume workload (1, 2 or 5)")
         wl.op = "agg"
     if a.v3 or a.feature:
-        if wl.op != "v1" or wl.storage not in (("f32",) if a.v3 else ("f32", "f64")):
+        if wl.op != "v1" or wl.storage not in ("f32", "f64"):
             sys.exit("bench.py: --v3 / --feature need a float32 CostVolume workload (1, 2 or 5)")
         wl.op = "v3" if a.v3 else "feat"
         wl.groups = a.v3 if a.v3 else 1

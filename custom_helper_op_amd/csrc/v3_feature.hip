@@ -163,34 +163,48 @@ __global__ __launch_bounds__(kBlock) void v3_forward_kernel(const Args<R> a) {
   }
 }
 
-// The D voxels of a pixel all add into the same ref_grad row and the same base-plane
-// gradient.  A workgroup covers kBlock consecutive voxels, i.e. a few consecutive pixels:
-// their rows are accumulated in LDS (ds_add) and leave as one global atomic per element and
-// workgroup.  LDS_ROWS = 0 selects plain global atomics (pixel rows that do not fit).
+// Thread -> voxel mapping of the gradient: the 64 lanes of a wave take 64 consecutive PIXELS
+// at one depth, the four waves of a workgroup four consecutive depths, and the workgroup walks
+// its segment of the depth range.  With the lanes along the depth axis (the reference's
+// order) all lanes of an atomic instruction add into the same few texels of src_grad;
+// neighbouring pixels hit neighbouring texels instead, and the rows of the pixel-owned
+// gradients (ref_grad, base-plane gradient: all D voxels of a pixel add into the same row)
+// are accumulated in LDS (ds_add) over the whole depth segment and leave as one global
+// atomic per element and workgroup.  lds_rows = 0 selects plain global atomics (rows that do
+// not fit).  What bounds the kernel either way is the number of source-gradient atomics, four
+// taps times the channels of a group per (voxel, view), one element each: 10.6 ms for the
+// gradient of the MVSNet-stage tensors (11.1 ms in the reference's order); the tiled kernels,
+// which merge them in registers and LDS first, take 0.5 ms for the shapes they cover.
+constexpr int kV3Pixels = 64, kV3Depths = kBlock / kV3Pixels;
 template <typename R, int REDUCE, int SUB>
-__global__ __launch_bounds__(kBlock) void v3_backward_kernel(const Args<R> a, int lds_rows) {
+__global__ __launch_bounds__(kBlock) void v3_backward_kernel(const Args<R> a, int lds_rows,
+                                                             int nsplit, int seg) {
   extern __shared__ __align__(16) unsigned char v3_smem[];
-  R *rows = reinterpret_cast<R *>(v3_smem);  // [lds_rows][C + 1]: ref_grad row, depth gradient
+  R *rows = reinterpret_cast<R *>(v3_smem);  // [64][C + 1]: ref_grad row, depth gradient
   const int C = (int)a.C, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW, D = (int)a.D;
   const int groups = a.groups, sub = C / groups;
-  const int64_t total = a.voxels();
+  const int64_t pixels = a.pixels();
   const int64_t row_step = (int64_t)srcW * C;
   const int RW = C + 1;
-  // every thread of a workgroup makes the same number of trips: the loop holds barriers
-  for (int64_t base = (int64_t)blockIdx.x * kBlock; base < total;
-       base += (int64_t)gridDim.x * kBlock) {
-    const int64_t pix0 = base / D;
-    if (lds_rows > 0) {
-      for (int k = threadIdx.x; k < lds_rows * RW; k += kBlock) rows[k] = R(0);
-      __syncthreads();
-    }
-    const int64_t i = base + threadIdx.x;
+  const int64_t group = (int64_t)blockIdx.x / nsplit;
+  const int split = (int)((int64_t)blockIdx.x - group * nsplit);
+  const int64_t pix0 = group * kV3Pixels;
+  const int lane_px = threadIdx.x % kV3Pixels, dw = threadIdx.x / kV3Pixels;
+  const int64_t pix = pix0 + lane_px;
+  const int d_lo = split * seg, d_hi = min(D, d_lo + seg);
+  if (lds_rows > 0) {
+    for (int k = threadIdx.x; k < kV3Pixels * RW; k += kBlock) rows[k] = R(0);
+    __syncthreads();
+  }
+  for (int d = d_lo + dw; d < d_hi; d += kV3Depths) {
+    if (pix >= pixels) break;
+    const int64_t i = pix * D + d;
     const int32_t *m = a.mask_in + (REDUCE == 0 ? i : i * 3);
-    const int32_t m0 = i < total ? m[0] : -1;
-    if (i < total && (REDUCE == 0 ? (m0 > 0) : (m0 >= 0))) {
+    const int32_t m0 = m[0];
+    if (REDUCE == 0 ? (m0 > 0) : (m0 >= 0)) {
       const Voxel<R> v = locate(a, i);
       const R *ref_px = a.ref + v.pix * C;
-      R *ref_lds = rows + (v.pix - pix0) * RW;  // (kept apart from the global row, so that
+      R *ref_lds = rows + lane_px * RW;         // (kept apart from the global row, so that
       R *ref_glb = a.ref_grad + v.pix * C;      //  the LDS adds compile to LDS instructions)
       // :426 cost_grad / (T)mask for the mean; the MIN gradient takes cost_grad as is (:621)
       const R cg = REDUCE == 0 ? a.cost_grad[i] / static_cast<R>(m0) : a.cost_grad[i];
@@ -241,20 +255,18 @@ __global__ __launch_bounds__(kBlock) void v3_backward_kernel(const Args<R> a, in
       else
         atomic_add(a.depth_grad + v.pix, depth_grad);
     }
-    if (lds_rows > 0) {
-      __syncthreads();
-      const int64_t pixels = a.pixels();
-      for (int k = threadIdx.x; k < lds_rows * RW; k += kBlock) {
-        const int r = k / RW, c = k - r * RW;
-        const R val = rows[k];
-        if (val != R(0) && pix0 + r < pixels) {
-          if (c < C)
-            atomic_add(a.ref_grad + (pix0 + r) * C + c, val);
-          else
-            atomic_add(a.depth_grad + pix0 + r, val);
-        }
+  }
+  if (lds_rows > 0) {
+    __syncthreads();
+    for (int k = threadIdx.x; k < kV3Pixels * RW; k += kBlock) {
+      const int r = k / RW, c = k - r * RW;
+      const R val = rows[k];
+      if (val != R(0) && pix0 + r < pixels) {
+        if (c < C)
+          atomic_add(a.ref_grad + (pix0 + r) * C + c, val);
+        else
+          atomic_add(a.depth_grad + pix0 + r, val);
       }
-      __syncthreads();
     }
   }
 }
@@ -375,14 +387,24 @@ hipError_t launch_v3_backward(const Args<S> &a, hipStream_t stream) {
   if ((err = zero.launch(stream)) != hipSuccess) return err;
   const int64_t total = a.voxels();
   if (total == 0 || a.C == 0) return hipSuccess;
-  const int grid = grid_for(total, kBlock);
   const int sub = v3_vector_width(a);
-  // pixels a workgroup's kBlock consecutive voxels can touch, and their rows in LDS
-  int lds_rows = (int)((kBlock + a.D - 1) / a.D) + 1;
+  // workgroups: groups of 64 pixels, times enough depth segments to give every SIMD a few
+  // waves (whole rounds of the four depths a workgroup covers at a time)
+  const int64_t pixel_groups = (a.pixels() + kV3Pixels - 1) / kV3Pixels;
+  int64_t nsplit = (256 * 4 * 2 + pixel_groups - 1) / pixel_groups;
+  const int64_t rounds = (a.D + kV3Depths - 1) / kV3Depths;
+  if (nsplit > rounds) nsplit = rounds;
+  if (nsplit < 1) nsplit = 1;
+  const int seg = (int)((rounds + nsplit - 1) / nsplit) * kV3Depths;
+  nsplit = (a.D + seg - 1) / seg;
+  if (pixel_groups * nsplit >= (int64_t)1 << 31) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)(pixel_groups * nsplit));
+  // the rows of the workgroup's pixels in LDS
+  int lds_rows = kV3Pixels;
   size_t smem = (size_t)lds_rows * (size_t)(a.C + 1) * sizeof(S);
   if (smem > 32 * 1024) lds_rows = 0, smem = 0;
 #define CHOP_V3_BWD(RED, SUB) \
-  v3_backward_kernel<S, RED, SUB><<<grid, kBlock, smem, stream>>>(a, lds_rows)
+  v3_backward_kernel<S, RED, SUB><<<grid, kBlock, smem, stream>>>(a, lds_rows, (int)nsplit, seg)
   if (a.reduce == 0) {
     if (sub == 8) CHOP_V3_BWD(0, 8); else if (sub == 4) CHOP_V3_BWD(0, 4); else CHOP_V3_BWD(0, 0);
   } else {
