@@ -43,6 +43,7 @@ SIGNATURES["chop_cost_volume_fwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] 
 SIGNATURES["chop_cost_volume_bwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 13 + [ctypes.c_size_t]
 SIGNATURES["chop_cost_volume_bwd_16_static"] = [_vp, _int, _int, _int] + _DIMS + [_vp] * 12
 SIGNATURES["chop_static_scratch_bytes"] = []
+SIGNATURES["chop_cost_default_fill_grad_16"] = [_vp, _int, _int, _i64, _i64] + [_vp] * 4
 SIGNATURES["chop_cost_volume_v2_fwd_16"] = [_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 7
 SIGNATURES["chop_cost_volume_v2_fwd_fill_16"] = [_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 8
 SIGNATURES["chop_cost_volume_v2_bwd_16"] = ([_vp, _int, _int, _int] + _DIMS + [_int] + [_vp] * 11

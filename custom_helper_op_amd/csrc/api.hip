@@ -670,6 +670,29 @@ int chop_cost_volume_bwd_16(void *stream, int storage, int reduce, int half_cent
                        (bf16_t *)src_grad, depth_grad, false, workspace, workspace_bytes))
 }
 
+int chop_cost_default_fill_grad_16(void *stream, int storage, int reduce, int64_t mask_count,
+                                   int64_t inner, const void *out_grad, const int32_t *mask,
+                                   void *cost_grad, float *default_grad) {
+  if (reduce != CHOP_REDUCE_MEAN && reduce != CHOP_REDUCE_MIN)
+    return fail(CHOP_ERR_BAD_ENUM, "reduce must be CHOP_REDUCE_MEAN (0) or CHOP_REDUCE_MIN (1)");
+  int64_t total;
+  if (mask_count < 0 || inner < 1 || mul_overflows({mask_count, inner}, &total))
+    return fail(CHOP_ERR_BAD_DIMS, "mask_count must be >= 0 and inner >= 1");
+  REQUIRE_PTR(default_grad, 1);
+  REQUIRE_PTR(out_grad, total);
+  REQUIRE_PTR(mask, total);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  STORAGE_DISPATCH(
+      launch_status(launch_default_fill_grad<__half>(reduce, mask_count, inner,
+                                                     (const __half *)out_grad, mask,
+                                                     (__half *)cost_grad, default_grad, s),
+                    "default fill gradient launch"),
+      launch_status(launch_default_fill_grad<bf16_t>(reduce, mask_count, inner,
+                                                     (const bf16_t *)out_grad, mask,
+                                                     (bf16_t *)cost_grad, default_grad, s),
+                    "default fill gradient launch"))
+}
+
 size_t chop_static_scratch_bytes(void) { return kScratchBytes; }
 
 int chop_cost_volume_bwd_16_static(void *stream, int storage, int reduce, int half_centor,

@@ -32,20 +32,20 @@ __global__ __launch_bounds__(kBlock) void default_fill_kernel(int reduce, int64_
   }
 }
 
-template <typename R>
+template <typename S, typename R>
 __global__ __launch_bounds__(kBlock) void default_fill_grad_kernel(int reduce, int64_t total,
                                                                    int64_t inner,
-                                                                   const R *out_grad,
+                                                                   const S *out_grad,
                                                                    const int32_t *mask,
-                                                                   R *cost_grad, R *default_grad) {
+                                                                   S *cost_grad, R *default_grad) {
   __shared__ R partial[kBlock / 64];
   R sum = R(0);
   for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total;
        e += (int64_t)gridDim.x * kBlock) {
     const int32_t m = mask[e / inner];
     const bool keep = reduce == 0 ? m > 0 : m >= 0;
-    const R g = out_grad[e];
-    if (cost_grad != nullptr) cost_grad[e] = keep ? g : R(0);
+    const R g = Storage<S>::load(out_grad + e);  // (16-bit storage: summed in float)
+    if (cost_grad != nullptr) Storage<S>::store(cost_grad + e, keep ? g : R(0));
     if (!keep) sum += g;
   }
   // wavefront sum, then one atomic per workgroup
@@ -139,17 +139,18 @@ hipError_t launch_default_fill(int reduce, int64_t mask_count, int64_t inner, co
   return hipGetLastError();
 }
 
-template <typename R>
+template <typename S>
 hipError_t launch_default_fill_grad(int reduce, int64_t mask_count, int64_t inner,
-                                    const R *out_grad, const int32_t *mask, R *cost_grad,
-                                    R *default_grad, hipStream_t stream) {
+                                    const S *out_grad, const int32_t *mask, S *cost_grad,
+                                    typename Storage<S>::Real *default_grad, hipStream_t stream) {
+  using R = typename Storage<S>::Real;
   hipError_t err = launch_fill_zero(default_grad, sizeof(R), stream);
   if (err != hipSuccess) return err;
   const int64_t total = mask_count * inner;
   if (total == 0) return hipSuccess;
   const int grid = (int)std::min<int64_t>(grid_for(total, kBlock), 2048);
-  default_fill_grad_kernel<R><<<grid, kBlock, 0, stream>>>(reduce, total, inner, out_grad, mask,
-                                                          cost_grad, default_grad);
+  default_fill_grad_kernel<S, R><<<grid, kBlock, 0, stream>>>(reduce, total, inner, out_grad, mask,
+                                                             cost_grad, default_grad);
   return hipGetLastError();
 }
 
@@ -173,5 +174,9 @@ hipError_t launch_combine_projection(int64_t B, int64_t N, const R *ref_cam, con
 CHOP_INSTANTIATE(float)
 CHOP_INSTANTIATE(double)
 #undef CHOP_INSTANTIATE
+template hipError_t launch_default_fill_grad<__half>(int, int64_t, int64_t, const __half *,
+                                                     const int32_t *, __half *, float *, hipStream_t);
+template hipError_t launch_default_fill_grad<bf16_t>(int, int64_t, int64_t, const bf16_t *,
+                                                     const int32_t *, bf16_t *, float *, hipStream_t);
 
 }  // namespace chop

@@ -24,6 +24,11 @@ enum Corr {
   WARP_ONLY = 4
 };
 
+// Dynamic LDS a workgroup may ask for at launch without any per-kernel attribute having been
+// set (HIP's limit on this hardware; the CU has 160 KiB).  Every kernel of the library stays
+// inside it, so the launchers keep no state and may run on any number of host threads.
+constexpr size_t kMaxDynamicLds = 64 * 1024;
+
 // Channels per group the CostVolumeV3 kernels hold in registers (MAX_SUBCHANNELS_SIZE,
 // custom_helper_op/cc/kernels/cost_volume_v3.h:35).
 constexpr int kMaxSubChannels = 8;
@@ -182,10 +187,11 @@ template <typename R>
 hipError_t launch_default_fill(int reduce, int64_t mask_count, int64_t inner, const R *cost,
                                const int32_t *mask, const R *default_cost, R *out,
                                hipStream_t stream);
-template <typename R>
+// (S: float, double, or a 16-bit storage type whose sum is kept in float)
+template <typename S>
 hipError_t launch_default_fill_grad(int reduce, int64_t mask_count, int64_t inner,
-                                    const R *out_grad, const int32_t *mask, R *cost_grad,
-                                    R *default_grad, hipStream_t stream);
+                                    const S *out_grad, const int32_t *mask, S *cost_grad,
+                                    typename Storage<S>::Real *default_grad, hipStream_t stream);
 template <typename R>
 hipError_t launch_combine_projection(int64_t B, int64_t N, const R *ref_cam, const R *src_cam,
                                      const R *scale, R *Rs, R *Ts, hipStream_t stream);

@@ -673,16 +673,20 @@ StripGeom strip_geometry(const Args<S> &a) {
   const int per = (int)((a.D + nseg - 1) / nseg);
   g.seg = (per + kDB - 1) / kDB * kDB;
   g.nseg = (int)((a.D + g.seg - 1) / g.seg);
-  // carried runs: N * 64 lanes * (4 sums + cell); given up beyond 16 KiB
-  g.carry = strip_run_bytes<S>(a.N) <= 16384;
-  // Wide pixels: the texel cache between the runs and memory, as long as
-  // it stays small (8 KiB: four views of 32 double-precision lanes) and a texel's index over
-  // all images of the call fits its 32-bit tag.
+  // carried runs: N * 64 lanes * (4 sums + tap offset + cell); given up beyond 16 KiB, or
+  // where records and runs together would pass the launch limit (one channel in float64:
+  // 39 KiB of records)
   using R = typename Storage<S>::Real;
-  // (float64 only: its atomics move twice the bytes; with 32-bit elements the cache's own
-  // work costs more than it saves, 749 against 735 us at 24 channels)
+  const size_t rec_bytes = strip_lds_bytes<R>(9, ppw * g.vg * kDB, 2);
+  g.carry = strip_run_bytes<S>(a.N) <= 16384 && rec_bytes + strip_run_bytes<S>(a.N) <= kMaxDynamicLds;
+  // Wide pixels in float64: the texel cache between the runs and memory, as long as it stays
+  // small (8 KiB: four views of 32 lanes) and a texel's index over all images of the call
+  // fits its 32-bit tag.  (float64 only: its atomics move twice the bytes; with 32-bit elements
+  // the cache's own work costs more than it saves, 749 against 735 us at 24 channels)
   g.cache = sizeof(R) == 8 && lpp >= 16 && strip_cache_bytes<R>(a.N, lpp) <= 8192 &&
-            a.B * a.N * a.srcH * a.srcW < (int64_t)1 << 31 && a.srcH < 32768 && a.srcW < 65536;
+            a.B * a.N * a.srcH * a.srcW < (int64_t)1 << 31 && a.srcH < 32768 && a.srcW < 65536 &&
+            rec_bytes + (g.carry ? strip_run_bytes<S>(a.N) : 0) + strip_cache_bytes<R>(a.N, lpp) <=
+                kMaxDynamicLds;
   return g;
 }
 

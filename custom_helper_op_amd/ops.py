@@ -551,18 +551,21 @@ class _CostAggregate(torch.autograd.Function):
 
 def _default_grad(grad_out, mask, reduce_method, like):
     """Gradient of the layers' scalar default: the upstream gradient summed over the voxels
-    that received it (one reduction kernel; the 16-bit storage types are widened first)."""
+    that received it (one reduction kernel; 16-bit storage is read as stored and summed in
+    float, without a widened copy)."""
     lib = _lib.load()
     red = _reduce_code(reduce_method)
     g = grad_out.contiguous()
-    if g.dtype in _STORAGE16:
-        g = g.float()
     n_mask = mask.numel()
     inner = g.numel() // n_mask if n_mask else 1
-    out = torch.empty((), dtype=g.dtype, device=g.device)
-    fn = (lib.chop_cost_default_fill_grad_f32 if g.dtype == torch.float32
-          else lib.chop_cost_default_fill_grad_f64)
-    _lib.check(fn(_stream(out), red, n_mask, inner, _ptr(g), _ptr(mask), None, _ptr(out)))
+    out = torch.empty((), dtype=_real_dtype(g.dtype), device=g.device)
+    if g.dtype in _STORAGE16:
+        _lib.check(lib.chop_cost_default_fill_grad_16(_stream(out), _STORAGE16[g.dtype], red, n_mask,
+                                                      inner, _ptr(g), _ptr(mask), None, _ptr(out)))
+    else:
+        fn = (lib.chop_cost_default_fill_grad_f32 if g.dtype == torch.float32
+              else lib.chop_cost_default_fill_grad_f64)
+        _lib.check(fn(_stream(out), red, n_mask, inner, _ptr(g), _ptr(mask), None, _ptr(out)))
     return out.to(like.dtype).reshape(like.shape)
 
 

@@ -278,6 +278,12 @@ int chop_cost_default_fill_grad_f64(void *stream, int reduce, int64_t mask_count
  * the intrinsic K in its upper-left 3x3) and scale [3] (multiplies the rows of both K; then
  * 0.5 is added to both principal points):
  *   R = src_K (src_R ref_R^T) ref_K^-1,   T = src_K (src_t - src_R ref_R^T ref_t). */
+/* The same for an upstream gradient in 16-bit storage (CHOP_STORAGE_F16 / _BF16), as the
+ * 16-bit CostVolumeV2 layer produces it: read as stored, summed in float; cost_grad (same
+ * storage type, may be NULL) as above. */
+int chop_cost_default_fill_grad_16(void *stream, int storage, int reduce, int64_t mask_count,
+                                   int64_t inner, const void *out_grad, const int32_t *mask,
+                                   void *cost_grad, float *default_grad);
 int chop_combine_projection_f32(void *stream, int64_t B, int64_t N, const float *ref_cam,
                                 const float *src_cam, const float *scale, float *Rs, float *Ts);
 int chop_combine_projection_f64(void *stream, int64_t B, int64_t N, const double *ref_cam,
