@@ -1,7 +1,7 @@
 // Tiled cost-volume kernels for gfx950 (MEAN and MIN / MAX reduces, every op of the family).
 //
 // Work decomposition.  A workgroup is one wavefront.  It owns PPW = 64/LPP pixels of one
-// image (two rows of PPW/2: a compact tile's samples change their texel cell together more
+// image (a compact block, see tile_rows: its samples change their texel cell together more
 // often than a long row's) and one contiguous segment of the D depth hypotheses; the LPP lanes
 // of a pixel each own VEC consecutive channels (C = LPP*VEC), so every tap read and every
 // cost-row write of a pixel is one contiguous C*sizeof(S) segment.  Depth runs innermost:
@@ -36,6 +36,14 @@
 namespace chop {
 namespace tiled {
 
+// Rows of a wave's pixel tile (PPW = 64 / LPP pixels, tile_rows x PPW / tile_rows): as square
+// as the pixel count allows.  The samples of a compact tile cross texel boundaries at more
+// nearly the same depths than those of a long row, so fewer wave iterations carry a cell
+// change (MVSNet-stage workload, 8 pixels: 0.49 of them for 2 x 4 against 0.61 for 1 x 8;
+// f16 cascade workload, 16 pixels: 0.49-0.68 per view for 4 x 4 against 0.57-0.75 for 2 x 8),
+// and its footprint in the source image has fewer texels per pixel.
+constexpr int tile_rows(int ppw) { return ppw >= 64 ? 8 : ppw >= 16 ? 4 : ppw >= 2 ? 2 : 1; }
+
 struct Geometry {
   int hw;                  // H*W
   int tiles_per_image;     // ceil(hw / PPW)
@@ -47,7 +55,7 @@ struct Geometry {
   int64_t units_per_xcd;   // ceil(total_units / 8)
   int xcd_shift;           // log2 of the units dealt to one XCD at a time; -1: one band per XCD
   int64_t grid;            // workgroups to launch
-  int tiles_x;             // tiles per image row (a tile: two rows of PPW/2 pixels)
+  int tiles_x;             // tiles per image row (a tile: tile_rows(PPW) rows of pixels)
   int sub;                 // channels per correlation group (1 for squared difference)
   // The last tiles of the launch are cut into shorter depth segments, so that the launch ends
   // on small workgroups instead of a last round of full-length ones on a half-empty chip.
@@ -325,14 +333,14 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
     t.pin = t_in;
     t.pix_ok = true;
   } else {
-    // A tile is two rows of PPW/2 pixels: the samples of a compact tile cross texel boundaries
+    // A tile is tile_rows(PPW) rows of pixels: the samples of a compact tile cross texel boundaries
     // at more nearly the same depths than those of a long row, so fewer wave iterations carry
     // a cell change (0.49 against 0.62 of them on the MVSNet-stage workload).  Tiles that
     // stick out of the image have their outside pixels switched off.
-    constexpr int TW = PPW / 2;
+    constexpr int TH = tile_rows(PPW), TW = PPW / TH;
     const int ty = t_in / g.tiles_x, tx = t_in - ty * g.tiles_x;
-    const int py = t.p >= TW ? 1 : 0;
-    const int y = ty * 2 + py, x = tx * TW + (t.p - py * TW);
+    const int py = t.p / TW;
+    const int y = ty * TH + py, x = tx * TW + (t.p - py * TW);
     t.pix_ok = y < (int)a.H && x < (int)a.W;
     t.pin = y * (int)a.W + x;
   }
@@ -1135,10 +1143,12 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
 template <int VEC, int LPP>
 struct Window {
   static constexpr int PPW = 64 / LPP;
-  // twice the tile's width (two rows of PPW/2 pixels) by eight rows: room for the samples'
-  // drift in either direction (against 4 x 2*PPW: 357 -> 338 us on the MVSNet-stage workload)
-  static constexpr int ROWS = 8;
-  static constexpr int COLS = PPW > 8 ? PPW : 8;
+  // twice the tile's height by twice its width, at least eight each way: room for the
+  // samples' drift in either direction (8 x 8 against 4 x 16 for the 2 x 4 pixels of 32
+  // channels: 357 -> 338 us on the MVSNet-stage workload)
+  static constexpr int TH = tile_rows(PPW), TW = PPW / TH;
+  static constexpr int ROWS = 2 * TH > 8 ? 2 * TH : 8;
+  static constexpr int COLS = 2 * TW > 8 ? 2 * TW : 8;
   static constexpr int SLOTS = ROWS * COLS;
   static_assert(SLOTS % 64 == 0, "window_move lists the slots 64 at a time");
   static constexpr int C = VEC * LPP;
@@ -1475,7 +1485,17 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 // Waves per SIMD the register budget is held to.  The kernel is latency-bound (its time
 // falls in proportion to the resident waves), so one view per workgroup at three waves
 // beats two views at two.
-constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 : nv <= 2 ? 2 : 1; }
+// Four lanes per pixel (16 channels), gradient of a mean: the window of its 4 x 4 pixel tile is
+// 4 KB, which leaves LDS for sixteen workgroups per CU, and the kernel needs 130 registers left
+// alone; held to 128 it spills three to five of them and the fourth wave takes the f16 cascade
+// workload from 300 to 268 us.  (The MIN / MAX gradients, which stage mask rows as well, and
+// the ops with one upstream value per voxel would spill 15 to 35 registers: three waves.)
+constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1) {
+  return nv == 1 && lpp == 4 && corr <= 1 && reduce == 0 ? 4
+         : nv == 1 && lpp <= 8                           ? 3
+         : nv <= 2                                       ? 2
+                                                         : 1;
+}
 
 // REDUCE: 0 gradient of the mean (mask = number of accepted views), 1 gradient of the
 // per-channel minimum / per-group maximum (mask = winning view per channel or group; a
@@ -1492,7 +1512,7 @@ constexpr int backward_waves(int nv, int lpp) { return nv == 1 && lpp <= 8 ? 3 :
 // registers they do not have (the 32-channel kernel spills with it).
 template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true,
           bool PV = (CORR == 1), bool VLOOP = false>
-__global__ __launch_bounds__(64, backward_waves(NV, LPP)) void backward_kernel(const Args<S> a,
+__global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
   using WN = Window<VEC, LPP>;
   constexpr int PPW = 64 / LPP;
@@ -2085,8 +2105,9 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
     g.tiles_x = (int)W;
     g.tiles_per_image = g.hw;
   } else {
-    g.tiles_x = (int)((W + PPW / 2 - 1) / (PPW / 2));
-    g.tiles_per_image = g.tiles_x * (int)((H + 1) / 2);
+    constexpr int TH = tile_rows(PPW), TW = PPW / TH;
+    g.tiles_x = (int)((W + TW - 1) / TW);
+    g.tiles_per_image = g.tiles_x * (int)((H + TH - 1) / TH);
   }
   const int64_t tiles = B * g.tiles_per_image;
   g.ngroups = ngroups;
