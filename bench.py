@@ -328,8 +328,10 @@ def other_configs(torch, lib, make_workload, skip_index, scratch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # (the defaults give the GPU's clocks time to settle: the first ~30 steps after an idle
+    # period run up to 15 % slower than the steady state)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true",

@@ -142,6 +142,12 @@ __device__ __forceinline__ void load_vec(const S *p, float *out) {
   }
 }
 
+// Output rows bypass the caches (non-temporal, STREAM) only where one store of a pixel's lanes covers
+// whole 128-byte lines.  A narrower row -- 16 channels of a 16-bit type, a few correlation
+// groups, the one mask word of a voxel -- shares its line with the rows of the neighbouring
+// depths, which other store instructions write: streamed, each piece reaches memory on its own
+// as a partial line, while L2 puts the pieces of a cached line together first (the
+// valid-view counts of the MVSNet-stage forward: 134 -> 123 us).
 template <typename S, int CNT, bool STREAM>
 __device__ __forceinline__ void store_vec(S *p, const float *in) {
   constexpr int BYTES = CNT * (int)sizeof(S);
@@ -197,6 +203,10 @@ __device__ __forceinline__ void widen_raw(const uint32_t *in, float *out) {
   }
 }
 
+// (the choice is made at compile time from the row's width: a run-time test in front of every
+// row store cost the MVSNet-stage forward 20 us)
+constexpr bool whole_lines(int elements, int elem_bytes) { return elements * elem_bytes >= 128; }
+
 // Orders this wave's LDS traffic: the lanes of a wavefront execute in lockstep and the
 // LDS returns a wave's operations in issue order, so only the compiler has to be kept
 // from moving accesses across the phase boundary.
@@ -251,17 +261,18 @@ __device__ __forceinline__ void fold_groups(const float *ch, int sub, float *out
   }
 }
 
-template <typename S, int VEC, bool STREAM>
+template <typename S, int VEC, int LPP>
 __device__ __forceinline__ void store_groups(S *p, const float *v, int sub) {
-  // p already points at this lane's first group
+  // p already points at this lane's first group; a pixel's row holds VEC * LPP / sub values
+  constexpr int C = VEC * LPP, B = (int)sizeof(S);
   if (sub == 1) {
-    store_vec<S, VEC, STREAM>(p, v);
+    store_vec<S, VEC, whole_lines(C, B)>(p, v);
   } else if (sub == 2) {
-    store_vec<S, VEC / 2, STREAM>(p, v);
+    store_vec<S, VEC / 2, whole_lines(C / 2, B)>(p, v);
   } else if (sub == 4) {
-    store_vec<S, VEC / 4, STREAM>(p, v);
+    store_vec<S, VEC / 4, whole_lines(C / 4, B)>(p, v);
   } else {
-    if constexpr (VEC >= 8) store_vec<S, VEC / 8, STREAM>(p, v);
+    if constexpr (VEC >= 8) store_vec<S, VEC / 8, whole_lines(C / 8, B)>(p, v);
   }
 }
 
@@ -414,19 +425,23 @@ __device__ __forceinline__ float voxel_depth(const Args<S> &a, int64_t pix, int 
 // =========================================================================================
 // Forward
 // =========================================================================================
-// Stores CNT (1, 2 or 4) consecutive int32 values, non-temporal.
-template <int CNT>
+// Stores CNT (1, 2 or 4) consecutive int32 values; STREAM as for the cost rows.
+template <int CNT, bool STREAM>
 __device__ __forceinline__ void store_ints(int32_t *p, const int *v) {
+  constexpr bool stream = STREAM;
   if constexpr (CNT == 4) {
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     i32x4 w = {v[0], v[1], v[2], v[3]};
-    __builtin_nontemporal_store(w, reinterpret_cast<i32x4 *>(p));
+    if (stream) __builtin_nontemporal_store(w, reinterpret_cast<i32x4 *>(p));
+    else *reinterpret_cast<i32x4 *>(p) = w;
   } else if constexpr (CNT == 2) {
     typedef int i32x2 __attribute__((ext_vector_type(2)));
     i32x2 w = {v[0], v[1]};
-    __builtin_nontemporal_store(w, reinterpret_cast<i32x2 *>(p));
+    if (stream) __builtin_nontemporal_store(w, reinterpret_cast<i32x2 *>(p));
+    else *reinterpret_cast<i32x2 *>(p) = w;
   } else {
-    __builtin_nontemporal_store(v[0], p);
+    if (stream) __builtin_nontemporal_store(v[0], p);
+    else *p = v[0];
   }
 }
 
@@ -617,6 +632,9 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
   // source group) as its mask (cost_volume_kernels_gpu_v3.cu.cc:52-146, :148-262)
   const int OC = CORR == 1 ? a.groups : (CORR == 2 || CORR == 3) ? 1 : C;
   const int gv = VEC / g.sub;  // output values per lane
+  // the cost rows of the per-channel ops (and the sample rows of the warp-only op) stream past
+  // the caches where they cover whole lines
+  constexpr bool kNtRows = whole_lines(VEC * LPP, (int)sizeof(S));
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   // the cost-map layers' default fill folded into the store: where no view was accepted the
   // scalar is written instead of the cost (custom_layers.py:52-57, :78-83)
@@ -645,7 +663,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
         if constexpr (CORR == 2 && REDUCE == 1) vmask |= (hit.off >= 0 ? 1u : 0u) << n;
         if constexpr (CORR == 4) {
           if (n < N && d_ok && t.pix_ok)
-            __builtin_nontemporal_store(hit.off >= 0 ? 1 : 0, a.mask + (t.pix * D + d) * N + n);
+            a.mask[(t.pix * D + d) * N + n] = hit.off >= 0 ? 1 : 0;
         }
         if constexpr (LPP > 1) {
           lds_at<int>(smem, q4, kOff + (n * LPP * PPW) * 4) = hit.off;
@@ -657,7 +675,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
         }
       }
       if constexpr (REDUCE == 0 && CORR != 4)
-        if (d_ok && t.pix_ok) __builtin_nontemporal_store(cnt, a.mask + t.pix * D + d);
+        if (d_ok && t.pix_ok) a.mask[t.pix * D + d] = cnt;
     }
     if constexpr (LPP > 1) wave_sync();
     if constexpr (CORR == 2 && REDUCE == 1) {
@@ -739,8 +757,8 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
       const int d = d0 + t.cl;
       if (d < d_hi && t.pix_ok) {
         const float out = win >= 0 ? best / static_cast<float>(C) : dflt;  // :222-227
-        __builtin_nontemporal_store(out, reinterpret_cast<float *>(a.cost) + t.pix * D + d);
-        __builtin_nontemporal_store(win, a.mask + t.pix * D + d);
+        reinterpret_cast<float *>(a.cost)[t.pix * D + d] = out;
+        a.mask[t.pix * D + d] = win;
       }
       continue;
     }
@@ -857,13 +875,13 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
               if (arg[jj][c] < 0) acc[jj][c] = dflt;
           }
           if (CORR == 0) {
-            store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
-            store_ints<VEC>(mout + t.cl * VEC, arg[jj]);
+            store_vec<S, VEC, kNtRows>(out + t.cl * VEC, acc[jj]);
+            store_ints<VEC, whole_lines(VEC * LPP, 4)>(mout + t.cl * VEC, arg[jj]);
           } else {
-            store_groups<S, VEC, true>(out + t.cl * gv, acc[jj], g.sub);
-            if (g.sub == 1) store_ints<VEC>(mout + t.cl * gv, arg[jj]);
-            else if (g.sub == 2) store_ints<VEC / 2>(mout + t.cl * gv, arg[jj]);
-            else store_ints<VEC / 4>(mout + t.cl * gv, arg[jj]);
+            store_groups<S, VEC, LPP>(out + t.cl * gv, acc[jj], g.sub);
+            if (g.sub == 1) store_ints<VEC, whole_lines(VEC * LPP, 4)>(mout + t.cl * gv, arg[jj]);
+            else if (g.sub == 2) store_ints<VEC / 2, whole_lines(VEC * LPP / 2, 4)>(mout + t.cl * gv, arg[jj]);
+            else store_ints<VEC / 4, whole_lines(VEC * LPP / 4, 4)>(mout + t.cl * gv, arg[jj]);
           }
         } else {
           if (kcnt[jj] > 1) {
@@ -876,7 +894,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
 #pragma unroll
               for (int c = 0; c < VEC; ++c) acc[jj][c] = dflt;
             }
-            store_vec<S, VEC, true>(out + t.cl * VEC, acc[jj]);
+            store_vec<S, VEC, kNtRows>(out + t.cl * VEC, acc[jj]);
           } else {
             float grp[VEC];
             fold_groups<VEC>(acc[jj], g.sub, grp);
@@ -884,7 +902,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
 #pragma unroll
               for (int c = 0; c < VEC; ++c) grp[c] = dflt;
             }
-            store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
+            store_groups<S, VEC, LPP>(out + t.cl * gv, grp, g.sub);
           }
         }
       }
@@ -980,7 +998,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
                        wt.w * tap[n][3][c];
           }
           if (n < N && t.pix_ok)
-            store_vec<S, VEC, true>(a.cost + ((t.pix * D + d) * N + n) * C + t.cl * VEC, smp);
+            store_vec<S, VEC, kNtRows>(a.cost + ((t.pix * D + d) * N + n) * C + t.cl * VEC, smp);
           continue;
         }
         if (off >= 0) {
@@ -1070,13 +1088,13 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
           S *out = out_pix + d * OC;  // d * OC is uniform: one add per lane
           int32_t *mout = mask_pix + d * OC;
           if (CORR == 0) {
-            store_vec<S, VEC, true>(out + t.cl * VEC, acc);
-            store_ints<VEC>(mout + t.cl * VEC, arg);
+            store_vec<S, VEC, kNtRows>(out + t.cl * VEC, acc);
+            store_ints<VEC, whole_lines(VEC * LPP, 4)>(mout + t.cl * VEC, arg);
           } else {
-            store_groups<S, VEC, true>(out + t.cl * gv, acc, g.sub);
-            if (g.sub == 1) store_ints<VEC>(mout + t.cl * gv, arg);
-            else if (g.sub == 2) store_ints<VEC / 2>(mout + t.cl * gv, arg);
-            else store_ints<VEC / 4>(mout + t.cl * gv, arg);
+            store_groups<S, VEC, LPP>(out + t.cl * gv, acc, g.sub);
+            if (g.sub == 1) store_ints<VEC, whole_lines(VEC * LPP, 4)>(mout + t.cl * gv, arg);
+            else if (g.sub == 2) store_ints<VEC / 2, whole_lines(VEC * LPP / 2, 4)>(mout + t.cl * gv, arg);
+            else store_ints<VEC / 4, whole_lines(VEC * LPP / 4, 4)>(mout + t.cl * gv, arg);
           }
         }
         continue;
@@ -1090,7 +1108,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
         if constexpr (LPP > 1) {
           if (t.cl == jj) agg_out = tot;
         } else {
-          if (t.pix_ok) __builtin_nontemporal_store(tot, reinterpret_cast<float *>(a.cost) + t.pix * D + d);
+          if (t.pix_ok) reinterpret_cast<float *>(a.cost)[t.pix * D + d] = tot;
         }
         continue;
       }
@@ -1106,7 +1124,7 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
 #pragma unroll
             for (int c = 0; c < VEC; ++c) acc[c] = dflt;
           }
-          store_vec<S, VEC, true>(out + t.cl * VEC, acc);
+          store_vec<S, VEC, kNtRows>(out + t.cl * VEC, acc);
         } else {
           float grp[VEC];
           fold_groups<VEC>(acc, g.sub, grp);
@@ -1114,13 +1132,13 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
 #pragma unroll
             for (int c = 0; c < VEC; ++c) grp[c] = dflt;
           }
-          store_groups<S, VEC, true>(out + t.cl * gv, grp, g.sub);
+          store_groups<S, VEC, LPP>(out + t.cl * gv, grp, g.sub);
         }
       }
     }
     if constexpr ((CORR == 2 || CORR == 3) && LPP > 1) {
       if (t.pix_ok && d0 + t.cl < d_hi)
-        __builtin_nontemporal_store(agg_out, reinterpret_cast<float *>(a.cost) + t.pix * D + d0 + t.cl);
+        reinterpret_cast<float *>(a.cost)[t.pix * D + d0 + t.cl] = agg_out;
     }
     if constexpr (CORR == 3 && REDUCE == 1) {
       if (t.pix_ok && d0 + t.cl < d_hi) {
@@ -1676,7 +1694,10 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
 #pragma unroll
           for (int jj = 0; jj < PF; ++jj) {
             const int d = min(first + jj, d_hi - 1);
-            load_vec<S, CNT, true>(cg_lane + (int64_t)d * cg_step, reinterpret_cast<float *>(cgw[jj]));
+            // (streamed past the caches only where a pixel's row covers whole lines: narrower
+            // rows share their line with the neighbouring depths' rows, which later loads want)
+            load_vec<S, CNT, whole_lines(CNT * LPP, (int)sizeof(S))>(
+                cg_lane + (int64_t)d * cg_step, reinterpret_cast<float *>(cgw[jj]));
           }
         };
         if (g.sub == 1) group_rows(std::integral_constant<int, VEC>());
@@ -1688,20 +1709,23 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
       for (int jj = 0; jj < PF; ++jj) {
         const int d = min(first + jj, d_hi - 1);
         const S *src_cg = cg_lane + (int64_t)d * cg_step;
-        if constexpr (CORR == 0 || CORR == 4) load_raw<S, VEC, true>(src_cg, cgw[jj]);
+        if constexpr (CORR == 0 || CORR == 4)
+          load_raw<S, VEC, whole_lines(VEC * LPP, (int)sizeof(S))>(src_cg, cgw[jj]);
         if constexpr (kMaskRows) {
           const int32_t *m = mask_lane + (int64_t)d * OC;
           const int cntv = CORR == 0 ? VEC : gv;
           if (cntv == 4) {
             typedef int i32x4 __attribute__((ext_vector_type(4)));
-            const i32x4 v = __builtin_nontemporal_load(reinterpret_cast<const i32x4 *>(m));
+            const i32x4 *q = reinterpret_cast<const i32x4 *>(m);
+            const i32x4 v = whole_lines(4 * LPP, 4) ? __builtin_nontemporal_load(q) : *q;
             mrow[jj][0] = v[0], mrow[jj][1] = v[1], mrow[jj][2] = v[2], mrow[jj][3] = v[3];
           } else if (cntv == 2) {
             typedef int i32x2 __attribute__((ext_vector_type(2)));
-            const i32x2 v = __builtin_nontemporal_load(reinterpret_cast<const i32x2 *>(m));
+            const i32x2 *q = reinterpret_cast<const i32x2 *>(m);
+            const i32x2 v = whole_lines(2 * LPP, 4) ? __builtin_nontemporal_load(q) : *q;
             mrow[jj][0] = v[0], mrow[jj][1] = v[1];
           } else {
-            mrow[jj][0] = __builtin_nontemporal_load(m);
+            mrow[jj][0] = whole_lines(LPP, 4) ? __builtin_nontemporal_load(m) : *m;
           }
         }
       }
