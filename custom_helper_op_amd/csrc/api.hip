@@ -234,6 +234,10 @@ int v3_call(void *stream, int reduce, int half_centor, const Dims &d, int groups
       }
     }
   }
+  if (g_kernel_family != 1 && work && backward && strip_pair_backward_supported(a)) {
+    g_last_family = 3;
+    return launch_status(launch_strip_backward(a, s), "strip CostVolumeV3 backward launch");
+  }
   g_last_family = 1;
   if (backward) return launch_status(launch_v3_backward(a, s), "CostVolumeV3 backward launch");
   return launch_status(launch_v3_forward(a, s), "CostVolumeV3 forward launch");

@@ -109,6 +109,9 @@ hipError_t launch_general_backward(const Args<S> &a, hipStream_t stream);
 // runs here.
 template <typename S>
 bool strip_supported(const Args<S> &a);
+// ... and the gradient of CostVolumeV3 (float, double; the forward pass has no strip kernel)
+template <typename S>
+bool strip_pair_backward_supported(const Args<S> &a);
 template <typename S>
 hipError_t launch_strip_forward(const Args<S> &a, hipStream_t stream);
 template <typename S>

@@ -2,7 +2,9 @@
 // not take -- float64 (the element type of the reference's own tests), channel counts that
 // are not 4 x a power of two (the reference tests use 3, 5 and 9), any number of views -- for
 // CostVolume, CostVolumeV2, CostAggregate (both reduces) and FeatureAggregate, all four storage
-// types, up to 64 channels.
+// types, up to 64 channels; and for the gradient of CostVolumeV3 in float and double with any
+// group width (the lanes of a pixel find the view's best group pair again through LDS, then
+// only the winning source group's lanes add into their taps).
 //
 // A workgroup is one wavefront.  It owns 64/LPP consecutive pixels (LPP = the power of two
 // >= C: one lane per channel, so a tap read or a cost-row write of a pixel is one contiguous
@@ -43,6 +45,7 @@ struct StripGeom {
   int vg;               // views reprojected together: min(N, max(1, LPP / kDB))
   int carry;            // backward: open runs survive the end of a chunk (in LDS)
   int cache;            // backward: a texel cache in LDS between the runs and memory
+  int pair_bytes;       // backward of CostVolumeV3: LDS of the group-pair search (0 otherwise)
   int64_t tiles;        // ceil(B*H*W / PPW)
 };
 
@@ -355,12 +358,15 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   const int C = (int)a.C, D = (int)a.D, N = (int)a.N, srcH = (int)a.srcH, srcW = (int)a.srcW;
   constexpr bool AGG = CORR == 2;   // CostAggregate: one upstream value per voxel
   constexpr bool FEAT = CORR == 4;  // FeatureAggregate: an upstream row and a mask entry per view
-  const int OC = CORR == 1 ? a.groups : AGG ? 1 : C;
-  const int sub = CORR == 1 ? C / a.groups : 1;
+  constexpr bool PAIR = CORR == 3;  // CostVolumeV3: one value per voxel, from the best group pair
+  const int OC = CORR == 1 ? a.groups : (AGG || PAIR) ? 1 : C;
+  const int MS = PAIR && REDUCE != 0 ? 3 : OC;  // mask entries per voxel (V3 MIN: view, two groups)
+  const int sub = (CORR == 1 || PAIR) ? C / a.groups : 1;
+  const int G = PAIR ? a.groups : 1;
   const int d_lo = segi * g.seg, d_hi = min(D, d_lo + g.seg);
   const StripPixel<R> px = strip_pixel(a, tile * ppw + p);
   const bool ch_ok = cl < C && px.ok;
-  const int oc = CORR == 1 ? (ch_ok ? cl / sub : 0) : AGG ? 0 : (ch_ok ? cl : 0);
+  const int oc = CORR == 1 ? (ch_ok ? cl / sub : 0) : (AGG || PAIR) ? 0 : (ch_ok ? cl : 0);
   const R ref_c = ch_ok && !FEAT ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
   const bool per_voxel = a.depth_grid != nullptr, want_depth = a.depth_grad != nullptr;
@@ -384,6 +390,13 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   if (cache)
     for (int k = lane; k < N * kCacheSlots; k += 64) s_tag[k] = -1;
   const unsigned long long pix_lanes = lpp == 64 ? ~0ull : ((1ull << lpp) - 1ull);
+  // CostVolumeV3: the pixel's reference row, the samples of the depth at hand and the dot
+  // products of all (source group, reference group) pairs, one set per pixel of the wave
+  R *s_ref = reinterpret_cast<R *>(reinterpret_cast<unsigned char *>(s_val) +
+                                   (cache ? strip_cache_bytes<R>(N, lpp) : 0));
+  R *s_smp = s_ref + 64, *s_dot = s_smp + 64;
+  const int my_group = PAIR && ch_ok ? cl / sub : -1, my_k = PAIR && ch_ok ? cl - my_group * sub : 0;
+  if constexpr (PAIR) s_ref[lane] = ref_c;
   const int64_t img_texels = (int64_t)srcH * srcW;
   R racc = R(0), dpart = R(0);
 
@@ -397,12 +410,15 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
     // its time in such waits).  They serve all views.
     R cgv[kDB];
     int win[REDUCE != 0 ? kDB : 1];
+    int win_gi[PAIR && REDUCE != 0 ? kDB : 1], win_gs[PAIR && REDUCE != 0 ? kDB : 1];
     if constexpr (!FEAT) {
 #pragma unroll
       for (int jj = 0; jj < kDB; ++jj) {
         const int64_t i = px.pix * D + min(d0 + jj, d_hi - 1);
         cgv[jj] = Storage<S>::load(a.cost_grad + i * OC + oc);
-        if constexpr (REDUCE != 0) win[jj] = a.mask_in[i * OC + oc];
+        if constexpr (REDUCE != 0) win[jj] = a.mask_in[i * MS + oc];
+        if constexpr (PAIR && REDUCE != 0)
+          win_gi[jj] = a.mask_in[i * MS + 1], win_gs[jj] = a.mask_in[i * MS + 2];
       }
     }
     for (int n0 = 0; n0 < N; n0 += g.vg) {
@@ -421,7 +437,7 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
         // memory once (mask, then depth, then camera, each behind a branch, were three waits)
         const int64_t i = px.pix * D + min(d, d_hi - 1);
         // FeatureAggregate: 1 / 0 per (voxel, view), :261-263
-        const int32_t m0 = FEAT ? a.mask_in[i * N + n0 + nl] : a.mask_in[REDUCE == 0 ? i : i * OC];
+        const int32_t m0 = FEAT ? a.mask_in[i * N + n0 + nl] : a.mask_in[REDUCE == 0 ? i : i * MS];
         const R dval = per_voxel ? a.depth_grid[i] : a.offsets[(int64_t)px.b * D + min(d, d_hi - 1)];
         R Rm[9], Tv[3];
 #pragma unroll
@@ -553,19 +569,58 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
             v00 = Storage<S>::load(q), v01 = Storage<S>::load(q + C);
             v11 = Storage<S>::load(q + C + row_step), v10 = Storage<S>::load(q + row_step);
           }
-          if (!ch_ok) continue;
+          if (!PAIR && !ch_ok) continue;
           if constexpr (REDUCE != 0)
             if (win[jj] != n) continue;  // another view won (:553)
           const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
                   k10 = rec.at(3, ridx + jj);
           const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
           const R cg = cgv[jj];
+          // CostVolumeV3 (cost_volume_kernels_gpu_v3.cu.cc:447-520, :593-640): the pair (reference
+          // group gi, source group gs) this view contributed -- searched again for the mean (source
+          // groups outermost, strict '<' from the smallest positive number, every dot product
+          // summed in channel order from zero: the order of the forward pass, so that the same
+          // pair wins), read from the mask for the MIN reduce.  All lanes of the pixel are here
+          // together: the samples go through LDS, lane q takes pair q.
+          int gi = -1, gs = -1;
+          if constexpr (PAIR) {
+            s_smp[lane] = ch_ok ? smp : R(0);
+            strip_sync();
+            if constexpr (REDUCE == 0) {
+              const int GG = G * G;
+              for (int q = cl; q < GG; q += lpp) {
+                const int qs = q / G, qi = q - qs * G;
+                R dot = R(0);
+                for (int k = 0; k < sub; ++k)
+                  dot += s_smp[p * lpp + qs * sub + k] * s_ref[p * lpp + qi * sub + k];
+                s_dot[p * GG + q] = dot;
+              }
+              strip_sync();
+              R best = Limits<R>::min_positive();
+              int bq = -1;
+              for (int q = 0; q < GG; ++q) {
+                const R dot = s_dot[p * GG + q];
+                if (best < dot) best = dot, bq = q;
+              }
+              // no pair above the seed: the reference indexes group -1 here (:495-496)
+              if (bq < 0) continue;
+              gs = bq / G, gi = bq - gs * G;
+            } else {
+              gi = win_gi[jj], gs = win_gs[jj];
+              if (gi < 0 || gi >= G || gs < 0 || gs >= G) continue;
+            }
+          }
           // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
           // reference's division (one division per voxel in phase 1 instead of one per element)
           const R inv = rec.at(8, ridx + jj);
           R gv;
           if constexpr (FEAT) {
             gv = cg;  // feature_aggregate_kernels_gpu.cu.cc:307-311
+          } else if constexpr (PAIR) {
+            const R scl = REDUCE == 0 ? cg * inv : cg;  // :426, :621
+            if (my_group == gi) racc += scl * s_smp[p * lpp + gs * sub + my_k];
+            if (my_group != gs) continue;  // only the winning source group receives a gradient
+            gv = scl * s_ref[p * lpp + gi * sub + my_k];
           } else if (CORR != 1) {
             const R diff = smp - ref_c;
             gv = (REDUCE == 0 || AGG) ? R(2) * diff * cg * inv : R(2) * diff * cg;  // :439, :560
@@ -677,7 +732,11 @@ StripGeom strip_geometry(const Args<S> &a) {
   // where records and runs together would pass the launch limit (one channel in float64:
   // 39 KiB of records)
   using R = typename Storage<S>::Real;
-  const size_t rec_bytes = strip_lds_bytes<R>(9, ppw * g.vg * kDB, 2);
+  // CostVolumeV3: 64 reference values, 64 samples, groups^2 dot products per pixel
+  g.pair_bytes = a.corr == BEST_GROUP_PAIR
+                     ? (int)((128 + (size_t)ppw * a.groups * a.groups) * sizeof(R))
+                     : 0;
+  const size_t rec_bytes = strip_lds_bytes<R>(9, ppw * g.vg * kDB, 2) + g.pair_bytes;
   g.carry = strip_run_bytes<S>(a.N) <= 16384 && rec_bytes + strip_run_bytes<S>(a.N) <= kMaxDynamicLds;
   // Wide pixels in float64: the texel cache between the runs and memory, as long as it stays
   // small (8 KiB: four views of 32 lanes) and a texel's index over all images of the call
@@ -703,6 +762,24 @@ bool strip_supported(const Args<S> &a) {
   if (a.srcH * a.srcW * a.C >= (int64_t)1 << 31) return false;  // 32-bit offsets inside a view
   const StripGeom g = strip_geometry(a);
   return g.tiles * g.nseg < (int64_t)1 << 31;
+}
+
+// The gradient of CostVolumeV3 in float and double: any group width (the general kernel, one
+// thread per voxel, sends every element of every tap to memory on its own).
+template <typename S>
+bool strip_pair_backward_supported(const Args<S> &a) {
+  if constexpr (sizeof(S) == 2) {
+    return false;
+  } else {
+    if (a.corr != BEST_GROUP_PAIR || a.depth_grid != nullptr) return false;
+    if (a.C < 1 || a.C > 64 || a.N < 1 || a.D < 1 || a.pixels() < 1) return false;
+    if (a.groups < 1 || a.C % a.groups != 0) return false;
+    if (a.srcH < 2 || a.srcW < 2) return false;
+    if (a.srcH * a.srcW * a.C >= (int64_t)1 << 31) return false;
+    const StripGeom g = strip_geometry(a);
+    if (g.pair_bytes > 16384) return false;  // very many groups: the search itself dominates
+    return g.tiles * g.nseg < (int64_t)1 << 31;
+  }
 }
 
 template <typename S>
@@ -756,9 +833,16 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
   if ((err = zero.launch(stream)) != hipSuccess) return err;
   const size_t smem = strip_lds_bytes<R>(9, (64 >> g.lpp_shift) * g.vg * kDB, 2) +
                       (g.carry ? strip_run_bytes<S>(a.N) : 0) +
-                      (g.cache ? strip_cache_bytes<R>(a.N, 1 << g.lpp_shift) : 0);
+                      (g.cache ? strip_cache_bytes<R>(a.N, 1 << g.lpp_shift) : 0) + g.pair_bytes;
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
-  if (a.corr == WARP_ONLY) {
+  if (a.corr == BEST_GROUP_PAIR) {
+    if constexpr (sizeof(S) != 2) {
+      if (a.reduce == 0)
+        strip_backward_kernel<S, 3, 0><<<grid, block, smem, stream>>>(a, g);
+      else
+        strip_backward_kernel<S, 3, 1><<<grid, block, smem, stream>>>(a, g);
+    }
+  } else if (a.corr == WARP_ONLY) {
     strip_backward_kernel<S, 4, 0><<<grid, block, smem, stream>>>(a, g);
   } else if (a.corr == SUM_SQUARED_DIFFERENCE) {
     if (a.reduce == 0)
@@ -787,6 +871,7 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
 
 #define CHOP_INSTANTIATE(S)                                                      \
   template bool strip_supported<S>(const Args<S> &);                             \
+  template bool strip_pair_backward_supported<S>(const Args<S> &);               \
   template hipError_t launch_strip_forward<S>(const Args<S> &, hipStream_t);     \
   template hipError_t launch_strip_backward<S>(const Args<S> &, hipStream_t);
 CHOP_INSTANTIATE(float)

@@ -87,10 +87,20 @@ def test_v3_backward(oracle, shape, reduce, dtype):
         _, mask = oracle.cost_volume_v3_fwd(*_args(t), reduce, G)
         cg = rng.normal(size=(B, H, W, D, 1)).astype(dtype)
         want = oracle.cost_volume_v3_bwd(*_args(t), cg, mask, reduce, G)
-        got = chop.cost_volume_grad_v3(*_inputs(t), dev(cg), dev(mask), reduce, G)
-        for g, w in zip(got, want):
-            assert g.shape == w.shape
-            assert_backward_close(host(g), w, rtol=1e-4 if dtype == np.float32 else 1e-10)
+        lib = _lib.load()
+        # the one-thread-per-voxel kernel, then the strip kernel (lane per channel: any group
+        # width, float and double), which is also what an unforced call picks for these shapes
+        # unless the tiled kernels take them
+        for family, ran in ((1, (1,)), (2, (3,)), (0, (2, 3))):
+            lib.chop_set_kernel_family(family)
+            try:
+                got = chop.cost_volume_grad_v3(*_inputs(t), dev(cg), dev(mask), reduce, G)
+                assert lib.chop_last_kernel_family() in ran
+            finally:
+                lib.chop_set_kernel_family(0)
+            for g, w in zip(got, want):
+                assert g.shape == w.shape
+                assert_backward_close(host(g), w, rtol=1e-4 if dtype == np.float32 else 1e-10)
 
 
 @pytest.mark.parametrize("C,G", [(8, 1), (8, 2), (16, 2), (16, 4), (32, 4), (32, 8), (64, 8),
@@ -165,14 +175,18 @@ def test_v3_tiled_ties(oracle, C, G):
         first = slice(0, sub) if variant == 0 else slice(sub, 2 * sub)
         outside = np.delete(want[0], np.r_[first], axis=-1)
         assert np.abs(want[0][..., first]).max() > 0 and not outside.any()
-        lib.chop_set_kernel_family(0)
-        got = chop.cost_volume_grad_v3(*_inputs(t), dev(cg), dev(mask), "MEAN", G)
-        assert lib.chop_last_kernel_family() == 2
-        assert_backward_close(host(got[0]), want[0])
-        assert_backward_close(host(got[1]), want[1])
-        # constant images: the depth gradient is exactly zero in the reference's form
-        # (differences of equal taps); the tiled kernel sums four weights that cancel
-        assert not want[2].any() and np.abs(host(got[2])).max() < 1e-6
+        for family, ran in ((0, 2), (2, 3)):   # tiled, then the strip kernel's search
+            lib.chop_set_kernel_family(family)
+            try:
+                got = chop.cost_volume_grad_v3(*_inputs(t), dev(cg), dev(mask), "MEAN", G)
+                assert lib.chop_last_kernel_family() == ran
+            finally:
+                lib.chop_set_kernel_family(0)
+            assert_backward_close(host(got[0]), want[0])
+            assert_backward_close(host(got[1]), want[1])
+            # constant images: the depth gradient is exactly zero in the reference's form
+            # (differences of equal taps); the tiled kernel sums four weights that cancel
+            assert not want[2].any() and np.abs(host(got[2])).max() < 1e-6
 
 
 def test_v3_backward_full_size(oracle):
@@ -186,6 +200,16 @@ def test_v3_backward_full_size(oracle):
         got = chop.cost_volume_grad_v3(*ins, dev(cg), mask, reduce, 4)
         assert _lib.load().chop_last_kernel_family() == 2
         want = oracle.cost_volume_v3_bwd(*_args(t), cg, host(mask), reduce, 4)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+        # the strip kernel (what float64 and other group widths run) on the same tensors
+        lib = _lib.load()
+        lib.chop_set_kernel_family(2)
+        try:
+            got = chop.cost_volume_grad_v3(*ins, dev(cg), mask, reduce, 4)
+            assert lib.chop_last_kernel_family() == 3
+        finally:
+            lib.chop_set_kernel_family(0)
         for g, w in zip(got, want):
             assert_backward_close(host(g), w)
 
