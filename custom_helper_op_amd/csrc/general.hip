@@ -212,22 +212,41 @@ __global__ __launch_bounds__(kBlock) void fill_zero_ranges_kernel(const ZeroRang
   for (int i = 0; i < r.count; ++i) zero_range(r.ptr[i], r.bytes[i]);
 }
 
+// fp32 accumulation images to their 16-bit outputs.  A thread takes eight consecutive elements:
+// two 16-byte loads that bypass the caches (an accumulator is read exactly once) and one
+// 16-byte store; with one element per thread the 2-byte stores held the pass to half the
+// stream rate.  `vec` = both pointers 16-byte aligned (else element by element).
 template <typename S>
-__global__ __launch_bounds__(kBlock) void narrow_kernel(const float *from, S *to, int64_t count) {
-  for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < count;
-       k += (int64_t)gridDim.x * kBlock)
-    Storage<S>::store(to + k, from[k]);
+__device__ __forceinline__ void narrow_range(const float *from, S *to, int64_t count, bool vec,
+                                             int64_t tid, int64_t stride) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  const int64_t octets = vec ? count / 8 : 0;
+  for (int64_t k = tid; k < octets; k += stride) {
+    const f32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(from) + 2 * k);
+    const f32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(from) + 2 * k + 1);
+    S out[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) Storage<S>::store(out + i, lo[i]), Storage<S>::store(out + 4 + i, hi[i]);
+    *(reinterpret_cast<u32x4 *>(to) + k) = *reinterpret_cast<const u32x4 *>(out);
+  }
+  for (int64_t k = octets * 8 + tid; k < count; k += stride) Storage<S>::store(to + k, from[k]);
+}
+
+template <typename S>
+__global__ __launch_bounds__(kBlock) void narrow_kernel(const float *from, S *to, int64_t count,
+                                                        bool vec) {
+  narrow_range<S>(from, to, count, vec, (int64_t)blockIdx.x * kBlock + threadIdx.x,
+                  (int64_t)gridDim.x * kBlock);
 }
 
 template <typename S>
 __global__ __launch_bounds__(kBlock) void narrow2_kernel(const float *from0, S *to0, int64_t count0,
-                                                         const float *from1, S *to1,
-                                                         int64_t count1) {
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < count0; k += stride)
-    Storage<S>::store(to0 + k, from0[k]);
-  for (int64_t k = (int64_t)blockIdx.x * kBlock + threadIdx.x; k < count1; k += stride)
-    Storage<S>::store(to1 + k, from1[k]);
+                                                         bool vec0, const float *from1, S *to1,
+                                                         int64_t count1, bool vec1) {
+  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
+  narrow_range<S>(from0, to0, count0, vec0, tid, stride);
+  narrow_range<S>(from1, to1, count1, vec1, tid, stride);
 }
 
 template <typename R>
@@ -281,13 +300,17 @@ hipError_t ZeroRanges::launch(hipStream_t stream) const {
   return hipGetLastError();
 }
 
+inline bool both_aligned16(const void *a, const void *b) {
+  return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+}
+
 template <typename S>
 hipError_t launch_narrow2(const float *from0, S *to0, int64_t count0, const float *from1, S *to1,
                           int64_t count1, hipStream_t stream) {
   const int64_t most = count0 > count1 ? count0 : count1;
   if (most == 0) return hipSuccess;
-  narrow2_kernel<S><<<grid_for(most, kBlock), kBlock, 0, stream>>>(from0, to0, count0, from1, to1,
-                                                                  count1);
+  narrow2_kernel<S><<<grid_for((most + 7) / 8, kBlock), kBlock, 0, stream>>>(
+      from0, to0, count0, both_aligned16(from0, to0), from1, to1, count1, both_aligned16(from1, to1));
   return hipGetLastError();
 }
 template hipError_t launch_narrow2<__half>(const float *, __half *, int64_t, const float *, __half *,
@@ -298,7 +321,8 @@ template hipError_t launch_narrow2<bf16_t>(const float *, bf16_t *, int64_t, con
 template <typename S>
 hipError_t launch_narrow(const float *from, S *to, int64_t count, hipStream_t stream) {
   if (count == 0) return hipSuccess;
-  narrow_kernel<S><<<grid_for(count, kBlock), kBlock, 0, stream>>>(from, to, count);
+  narrow_kernel<S><<<grid_for((count + 7) / 8, kBlock), kBlock, 0, stream>>>(from, to, count,
+                                                                             both_aligned16(from, to));
   return hipGetLastError();
 }
 template hipError_t launch_narrow<__half>(const float *, __half *, int64_t, hipStream_t);
