@@ -57,11 +57,6 @@ struct Geometry {
   int64_t grid;            // workgroups to launch
   int tiles_x;             // tiles per image row (a tile: tile_rows(PPW) rows of pixels)
   int sub;                 // channels per correlation group (1 for squared difference)
-  // The last tiles of the launch are cut into shorter depth segments, so that the launch ends
-  // on small workgroups instead of a last round of full-length ones on a half-empty chip.
-  int tail_tile0;          // first tile of the tail (== all tiles: no tail)
-  unsigned tail_unit0;     // its first unit
-  int tail_nseg, tail_seg; // depth segments of a tail tile
   float src_h_max, src_w_max;  // (float)(srcH - 1), (float)(srcW - 1): acceptance bounds
 };
 
@@ -325,17 +320,13 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
   if (unit >= (unsigned)g.total_units) return false;
   // the groups of one (tile, segment) are neighbours in launch order: they stream the same
   // upstream-gradient rows at about the same time, through the same L2
-  const bool tail = unit >= g.tail_unit0;
-  const unsigned per_tile = (unsigned)((tail ? g.tail_nseg : g.nseg) * g.ngroups);
-  const unsigned u = tail ? unit - g.tail_unit0 : unit;
-  const unsigned tile_in = u / per_tile;
-  const unsigned tile = tile_in + (tail ? (unsigned)g.tail_tile0 : 0u);
-  const int rem = (int)(u - tile_in * per_tile);
+  const unsigned per_tile = (unsigned)(g.nseg * g.ngroups);
+  const unsigned tile = unit / per_tile;
+  const int rem = (int)(unit - tile * per_tile);
   const int segi = rem / g.ngroups;
-  const int seg_len = tail ? g.tail_seg : g.seg;
   t.view0 = (rem - segi * g.ngroups) * g.vper;
-  t.d_lo = segi * seg_len;
-  t.d_hi = min((int)a.D, t.d_lo + seg_len);
+  t.d_lo = segi * g.seg;
+  t.d_hi = min((int)a.D, t.d_lo + g.seg);
   t.b = (int)(tile / (unsigned)g.tiles_per_image);
   const int t_in = (int)(tile - (unsigned)t.b * (unsigned)g.tiles_per_image);
   t.p = t.lane / LPP;
@@ -2117,16 +2108,13 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
   // pixel-owned gradients: one store when this workgroup saw every depth, otherwise one
   // atomic add per depth segment into the zero-filled outputs
   float *rg = kWide ? a.ref_grad_acc : reinterpret_cast<float *>(a.ref_grad);
-  const bool single = g.nseg * g.ngroups == 1;  // (such a launch has no tail: add_tail)
+  const bool single = g.nseg * g.ngroups == 1;
   if constexpr (CORR == 4) {
     // no reference image, no gradient for it
   } else if (single) {
-    if (t.pix_ok) {
-      if (kWide)
-        store_vec<float, VEC, false>(rg + t.pix * C + t.cl * VEC, racc);
-      else
-        store_vec<S, VEC, false>(a.ref_grad + t.pix * C + t.cl * VEC, racc);
-    }
+    // (16-bit storage too: the finished sums go straight to the output, the fp32 image of
+    // ref_grad is neither written nor narrowed afterwards)
+    if (t.pix_ok) store_vec<S, VEC, false>(a.ref_grad + t.pix * C + t.cl * VEC, racc);
   } else if (t.pix_ok) {
 #pragma unroll
     for (int c = 0; c < VEC; ++c) atomic_add(rg + t.pix * C + t.cl * VEC + c, racc[c]);
@@ -2155,13 +2143,6 @@ inline int choose_segments(int64_t tiles, int64_t D, int lpp, int64_t target_uni
   return nseg;
 }
 
-inline void size_grid(Geometry &g) {
-  g.units_per_xcd = (g.total_units + 7) / 8;
-  const int64_t round_to = g.xcd_shift >= 0 ? (int64_t)8 << g.xcd_shift : 8;
-  g.grid = g.xcd_shift >= 0 ? (g.total_units + round_to - 1) / round_to * round_to
-                            : g.units_per_xcd * 8;
-}
-
 template <int LPP>
 inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int sub, int ngroups = 1,
                               int vper = 0) {
@@ -2185,35 +2166,16 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   g.seg = ((per_seg + LPP - 1) / LPP) * LPP;
   g.nseg = (int)((D + g.seg - 1) / g.seg);
   g.total_units = tiles * g.nseg * g.ngroups;
-  g.tail_tile0 = (int)tiles;
-  g.tail_unit0 = (unsigned)g.total_units;
-  g.tail_nseg = g.nseg;
-  g.tail_seg = g.seg;
   // backward: runs of 32 units (the view groups of a tile are neighbours and mostly share
   // a run, hence an L2)
   g.xcd_shift = vper > 0 ? 5 : -1;
-  size_grid(g);
+  g.units_per_xcd = (g.total_units + 7) / 8;
+  const int64_t round_to = g.xcd_shift >= 0 ? (int64_t)8 << g.xcd_shift : 8;
+  g.grid = g.xcd_shift >= 0 ? (g.total_units + round_to - 1) / round_to * round_to
+                            : g.units_per_xcd * 8;
   g.sub = sub;
   g.src_h_max = g.src_w_max = 0.f;  // set by the launcher from the source image size
   return g;
-}
-
-// Cuts the last `tail_tiles` tiles of a launch whose units are dealt to the XCDs in short
-// runs (the backward) into depth segments `factor` times shorter.  Only for launches whose
-// pixel-owned outputs are accumulated anyway (more than one workgroup per pixel tile).
-template <int LPP>
-inline void add_tail(Geometry &g, int64_t tiles, int64_t D, int64_t tail_tiles, int factor) {
-  if (g.xcd_shift < 0 || g.nseg * g.ngroups == 1 || tail_tiles <= 0 || factor < 2) return;
-  if (tail_tiles > tiles) tail_tiles = tiles;
-  int seg2 = ((g.seg / factor + LPP - 1) / LPP) * LPP;
-  if (seg2 < LPP) seg2 = LPP;
-  if (seg2 >= g.seg) return;
-  g.tail_tile0 = (int)(tiles - tail_tiles);
-  g.tail_unit0 = (unsigned)((int64_t)g.tail_tile0 * g.nseg * g.ngroups);
-  g.tail_seg = seg2;
-  g.tail_nseg = (int)((D + seg2 - 1) / seg2);
-  g.total_units = (int64_t)g.tail_unit0 + tail_tiles * g.tail_nseg * g.ngroups;
-  size_grid(g);
 }
 
 template <typename S>
