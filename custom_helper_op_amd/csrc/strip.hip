@@ -390,11 +390,10 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   if (cache)
     for (int k = lane; k < N * kCacheSlots; k += 64) s_tag[k] = -1;
   const unsigned long long pix_lanes = lpp == 64 ? ~0ull : ((1ull << lpp) - 1ull);
-  // CostVolumeV3: the pixel's reference row, the samples of the depth at hand and the dot
-  // products of all (source group, reference group) pairs, one set per pixel of the wave
+  // CostVolumeV3: the pixels' reference rows and the samples of the depth at hand
   R *s_ref = reinterpret_cast<R *>(reinterpret_cast<unsigned char *>(s_val) +
                                    (cache ? strip_cache_bytes<R>(N, lpp) : 0));
-  R *s_smp = s_ref + 64, *s_dot = s_smp + 64;
+  R *s_smp = s_ref + 64;
   const int my_group = PAIR && ch_ok ? cl / sub : -1, my_k = PAIR && ch_ok ? cl - my_group * sub : 0;
   if constexpr (PAIR) s_ref[lane] = ref_c;
   const int64_t img_texels = (int64_t)srcH * srcW;
@@ -581,26 +580,29 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
           // groups outermost, strict '<' from the smallest positive number, every dot product
           // summed in channel order from zero: the order of the forward pass, so that the same
           // pair wins), read from the mask for the MIN reduce.  All lanes of the pixel are here
-          // together: the samples go through LDS, lane q takes pair q.
+          // together: the samples go through LDS.
           int gi = -1, gs = -1;
           if constexpr (PAIR) {
             s_smp[lane] = ch_ok ? smp : R(0);
             strip_sync();
             if constexpr (REDUCE == 0) {
+              // lane cl takes the pairs cl, cl + LPP, ... in ascending order, then the pixel's
+              // lanes compare: the larger product wins, of two equal ones the earlier pair --
+              // which is what the reference's scan with '<' keeps
               const int GG = G * G;
+              R best = Limits<R>::min_positive();
+              int bq = -1;
               for (int q = cl; q < GG; q += lpp) {
                 const int qs = q / G, qi = q - qs * G;
                 R dot = R(0);
                 for (int k = 0; k < sub; ++k)
                   dot += s_smp[p * lpp + qs * sub + k] * s_ref[p * lpp + qi * sub + k];
-                s_dot[p * GG + q] = dot;
-              }
-              strip_sync();
-              R best = Limits<R>::min_positive();
-              int bq = -1;
-              for (int q = 0; q < GG; ++q) {
-                const R dot = s_dot[p * GG + q];
                 if (best < dot) best = dot, bq = q;
+              }
+              for (int sh = 0; sh < g.lpp_shift; ++sh) {
+                const R ov = __shfl_xor(best, 1 << sh, 64);
+                const int oq = __shfl_xor(bq, 1 << sh, 64);
+                if (ov > best || (ov == best && oq >= 0 && oq < bq)) best = ov, bq = oq;
               }
               // no pair above the seed: the reference indexes group -1 here (:495-496)
               if (bq < 0) continue;
@@ -732,10 +734,8 @@ StripGeom strip_geometry(const Args<S> &a) {
   // where records and runs together would pass the launch limit (one channel in float64:
   // 39 KiB of records)
   using R = typename Storage<S>::Real;
-  // CostVolumeV3: 64 reference values, 64 samples, groups^2 dot products per pixel
-  g.pair_bytes = a.corr == BEST_GROUP_PAIR
-                     ? (int)((128 + (size_t)ppw * a.groups * a.groups) * sizeof(R))
-                     : 0;
+  // CostVolumeV3: 64 reference values and 64 samples
+  g.pair_bytes = a.corr == BEST_GROUP_PAIR ? (int)(128 * sizeof(R)) : 0;
   const size_t rec_bytes = strip_lds_bytes<R>(9, ppw * g.vg * kDB, 2) + g.pair_bytes;
   g.carry = strip_run_bytes<S>(a.N) <= 16384 && rec_bytes + strip_run_bytes<S>(a.N) <= kMaxDynamicLds;
   // Wide pixels in float64: the texel cache between the runs and memory, as long as it stays
@@ -777,7 +777,7 @@ bool strip_pair_backward_supported(const Args<S> &a) {
     if (a.srcH < 2 || a.srcW < 2) return false;
     if (a.srcH * a.srcW * a.C >= (int64_t)1 << 31) return false;
     const StripGeom g = strip_geometry(a);
-    if (g.pair_bytes > 16384) return false;  // very many groups: the search itself dominates
+    if (a.groups > 16) return false;  // very many groups: the search of groups^2 pairs dominates
     return g.tiles * g.nseg < (int64_t)1 << 31;
   }
 }
