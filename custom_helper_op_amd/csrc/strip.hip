@@ -612,8 +612,9 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
               if (gi < 0 || gi >= G || gs < 0 || gs >= G) continue;
             }
           }
-          // 1 / (views accepted): exact for 1, 2 and 4 views, else within one rounding of the
-          // reference's division (one division per voxel in phase 1 instead of one per element)
+          // 1 / (views accepted): exact for 1, 2 and 4 views, else within an ulp or two of the
+          // reference's division (one reciprocal per voxel in phase 1 instead of a division
+          // per element)
           const R inv = rec.at(8, ridx + jj);
           R gv;
           if constexpr (FEAT) {

@@ -1,8 +1,10 @@
 // TensorFlow-side shim: keeps the op registrations of zhuimeng999/custom_helper_op's
 // cost-volume family and turns each OpKernel into a call of libchop_costvol's C ABI.
 //
-// It is NOT built in this repository's image (no TensorFlow headers exist here); build it
-// where a ROCm TensorFlow is installed:
+// No TensorFlow exists in this repository's image: here the file only passes the compiler's
+// syntax and type check against stand-in headers that declare the few TensorFlow classes it
+// uses (tests/test_shim_compile.py, tests/tf_stubs/).  Build it where a ROCm TensorFlow is
+// installed:
 //   hipcc/g++ -std=c++17 -shared -fPIC cost_volume_ops.cc -I<repo>/include \
 //       $(python -c 'import tensorflow as tf; print(" ".join(tf.sysconfig.get_compile_flags()))') \
 //       $(python -c 'import tensorflow as tf; print(" ".join(tf.sysconfig.get_link_flags()))') \

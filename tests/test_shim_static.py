@@ -1,6 +1,7 @@
 """Static check of the TensorFlow shim (custom_helper_op_amd/tf_shim/cost_volume_ops.cc).
-No TensorFlow exists in this image, so no compiler ever sees the shim; every pointer argument
-of a forwarding overload has the same type, so a transposed argument would compile anywhere.
+No TensorFlow exists in this image (test_shim_compile.py runs the compiler's syntax check
+against stand-in headers); every pointer argument of a forwarding overload has the same type,
+so a transposed argument would compile anywhere.
 This test parses the overloads and the prototypes of include/chop_costvol.h and checks, per
 call: the callee exists, the arity agrees, every argument's type equals the prototype's
 parameter type, and the pointer arguments are forwarded in the order the overload received
