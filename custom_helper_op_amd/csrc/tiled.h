@@ -1199,10 +1199,27 @@ struct Window {
   // samples' drift in either direction (8 x 8 against 4 x 16 for the 2 x 4 pixels of 32
   // channels: 357 -> 338 us on the MVSNet-stage workload)
   static constexpr int TH = tile_rows(PPW), TW = PPW / TH;
-  static constexpr int ROWS = 2 * TH > 8 ? 2 * TH : 8;
+  // Eight lanes per pixel (32 channels, 2 x 4 pixels): six rows instead of eight.  With a
+  // 6 KB window the workgroup's LDS is 10 KB, so that sixteen workgroups fit a CU (four waves
+  // per SIMD: see backward_waves); four rows measured 2 % slower than eight at equal
+  // occupancy, six sit between.  The ring index of a row is then a remainder, not a mask.
+  static constexpr int ROWS = LPP == 8 ? 6 : (2 * TH > 8 ? 2 * TH : 8);
   static constexpr int COLS = 2 * TW > 8 ? 2 * TW : 8;
   static constexpr int SLOTS = ROWS * COLS;
-  static_assert(SLOTS % 64 == 0, "window_move lists the slots 64 at a time");
+  static constexpr bool kPow2Rows = (ROWS & (ROWS - 1)) == 0;
+  // ring row of image row `fh` (not negative)
+  static __device__ __forceinline__ int ring_row(unsigned fh) {
+    return kPow2Rows ? (int)(fh & (unsigned)(ROWS - 1)) : (int)(fh % (unsigned)ROWS);
+  }
+  // image row of ring row `ry` for a window whose first row is `oy` (any sign)
+  static __device__ __forceinline__ int image_row(int ry, int oy) {
+    if constexpr (kPow2Rows) {
+      return oy + ((ry - oy) & (ROWS - 1));
+    } else {
+      int m = (ry - oy) % ROWS;
+      return oy + (m < 0 ? m + ROWS : m);
+    }
+  }
   static constexpr int C = VEC * LPP;
   static constexpr int STRIDE = C;      // one slot = C consecutive words: 16-byte lane accesses
   static constexpr int kNone = 0x3fffffff;
@@ -1212,7 +1229,7 @@ struct Window {
   // slots of the taps 00, 01, 11, 10 of cell `key`, one byte each
   static __device__ __forceinline__ unsigned pack_slots(int key) {
     const int fh = (key >> 16) & 0x7fff, fw = key & 0xffff;
-    const int ry0 = (fh & (ROWS - 1)) * COLS, ry1 = ((fh + 1) & (ROWS - 1)) * COLS;
+    const int ry0 = ring_row((unsigned)fh) * COLS, ry1 = ring_row((unsigned)fh + 1u) * COLS;
     const int rx0 = fw & (COLS - 1), rx1 = (fw + 1) & (COLS - 1);
     return (unsigned)(ry0 + rx0) | ((unsigned)(ry0 + rx1) << 8) | ((unsigned)(ry1 + rx1) << 16) |
            ((unsigned)(ry1 + rx0) << 24);
@@ -1273,11 +1290,11 @@ __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, fl
     wave_sync();  // the adds of the chunk before are complete and visible
     int count = 0;
     for (int sb = 0; sb < WN::SLOTS; sb += 64) {
-      const int s = sb + lane;
+      const int s = sb + lane;  // (a window of 48 slots: the last lanes have none)
       const int ry = s / WN::COLS, rx = s % WN::COLS;
-      const int y = oy + ((ry - oy) & (WN::ROWS - 1)), x = ox + ((rx - ox) & (WN::COLS - 1));
-      const bool leaving = !((unsigned)(y - ny) < (unsigned)WN::ROWS &&
-                             (unsigned)(x - nx) < (unsigned)WN::COLS);
+      const int y = WN::image_row(ry, oy), x = ox + ((rx - ox) & (WN::COLS - 1));
+      const bool leaving = s < WN::SLOTS && !((unsigned)(y - ny) < (unsigned)WN::ROWS &&
+                                              (unsigned)(x - nx) < (unsigned)WN::COLS);
       const unsigned long long m = __ballot(leaving);
       if (leaving) {
         const int rank = count + (int)__builtin_amdgcn_mbcnt_hi(
@@ -1360,7 +1377,7 @@ __device__ __forceinline__ void window_flush_all(int oy, int ox, const float *da
         const int e = (i0 + u) * 64 + lane;  // float index inside the window
         const int sl = e / C, ch = e - sl * C;
         const int ry = sl / WN::COLS, rx = sl - ry * WN::COLS;
-        const int y = oy + ((ry - oy) & (WN::ROWS - 1)), x = ox + ((rx - ox) & (WN::COLS - 1));
+        const int y = WN::image_row(ry, oy), x = ox + ((rx - ox) & (WN::COLS - 1));
         if (v[u] != 0.f) atomic_add(gview + ((int64_t)(y * srcW + x) * C + ch), v[u]);
       }
     }
@@ -1369,7 +1386,7 @@ __device__ __forceinline__ void window_flush_all(int oy, int ox, const float *da
 #pragma unroll 1
   for (int ry = 0; ry < WN::ROWS; ++ry) {
     if (!((rows >> ry) & 1u)) continue;  // uniform
-    const int y = oy + ((ry - oy) & (WN::ROWS - 1));
+    const int y = WN::image_row(ry, oy);
     float v[PER_ROW];
 #pragma unroll
     for (int u = 0; u < PER_ROW; ++u) v[u] = data[(ry * PER_ROW + u) * 64 + lane];
@@ -1398,7 +1415,7 @@ __device__ __forceinline__ void window_flush_all(int oy, int ox, const float *da
 // from 429 to 400 us; against LDS atomics it halved the time of the 8-channel workloads.
 // 16 lanes per pixel (four pixels per wave): the pixels that fire in the same instruction
 // take turns, one pixel per round with its four taps in flight together.
-template <int VEC, int LPP>
+template <int VEC, int LPP, bool LEAN = false>
 __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4][VEC],
                                            float *data, int *tags, int lane, int cl) {
   using WN = Window<VEC, LPP>;
@@ -1412,7 +1429,7 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
       slot[3] = slots >> 24;
     } else {
       const int fh = (key >> 16) & 0x7fff, fw = key & 0xffff;
-      const int ry0 = (fh & (WN::ROWS - 1)) * WN::COLS, ry1 = ((fh + 1) & (WN::ROWS - 1)) * WN::COLS;
+      const int ry0 = WN::ring_row((unsigned)fh) * WN::COLS, ry1 = WN::ring_row((unsigned)fh + 1u) * WN::COLS;
       const int rx0 = fw & (WN::COLS - 1), rx1 = (fw + 1) & (WN::COLS - 1);
       slot[0] = ry0 + rx0, slot[1] = ry0 + rx1, slot[2] = ry1 + rx1, slot[3] = ry1 + rx0;
     }
@@ -1441,16 +1458,27 @@ __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4
       bool pending = true;
       if (__popcll(__ballot(true)) == LPP) {
         // one pixel alone (four of ten events on the headline workload): nothing to
-        // collide with, its four taps go in flight together
-        vecf old[4];
+        // collide with, its four taps go in flight together -- or, in a kernel held to a
+        // register budget, one after the other (twelve registers less at the kernel's peak)
+        if constexpr (LEAN) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-          old[k] = *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE);
+          for (int k = 0; k < 4; ++k) {
+            vecf old = *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+            for (int i = 0; i < VEC; ++i) old[i] += v[k][i];
+            *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE) = old;
+          }
+        } else {
+          vecf old[4];
 #pragma unroll
-          for (int i = 0; i < VEC; ++i) old[k][i] += v[k][i];
-          *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE) = old[k];
+          for (int k = 0; k < 4; ++k)
+            old[k] = *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) old[k][i] += v[k][i];
+            *reinterpret_cast<vecf *>(base + slot[k] * WN::STRIDE) = old[k];
+          }
         }
         pending = false;
       }
@@ -1542,8 +1570,19 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 // alone; held to 128 it spills three to five of them and the fourth wave takes the f16 cascade
 // workload from 300 to 268 us.  (The MIN / MAX gradients, which stage mask rows as well, and
 // the ops with one upstream value per voxel would spill 15 to 35 registers: three waves.)
+// Eight lanes per pixel (32 channels), gradient of the mean squared difference: 161 registers
+// left alone.  Held to 128 it spills 80 bytes in the depth loop, so the kernel is slimmed
+// first (lean_backward): four upstream rows staged at a time instead of eight (16 registers),
+// the records of a depth read where the depth starts instead of one depth ahead (10), the
+// four window taps of a pixel that fires alone added one after the other (12) -- 127 registers,
+// no scratch.  Those three cost 5 % at three waves per SIMD; with the 10 KB of LDS of the
+// six-row window the fourth wave gains 11 %.
+constexpr bool lean_backward(int nv, int lpp, int corr, int reduce) {
+  return nv == 1 && lpp == 8 && corr == 0 && reduce == 0;
+}
 constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1) {
-  return nv == 1 && lpp == 4 && corr <= 1 && reduce == 0 ? 4
+  return lean_backward(nv, lpp, corr, reduce)              ? 4
+         : nv == 1 && lpp == 4 && corr <= 1 && reduce == 0 ? 4
          : nv == 1 && lpp <= 8                           ? 3
          : nv <= 2                                       ? 2
                                                          : 1;
@@ -1622,7 +1661,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   // upstream-gradient rows fetched ahead; the MIN reduce stages the mask rows beside them
-  constexpr int PFMAX = REDUCE ? 4 : 8;
+  constexpr bool kLean = lean_backward(NV, LPP, CORR, REDUCE) && !VLOOP;
+  constexpr int PFMAX = (REDUCE || kLean) ? 4 : 8;
   constexpr int PF = LPP < PFMAX ? LPP : PFMAX;
   constexpr bool kMaskRows = REDUCE == 1 && !kVoxelGrad;
   // mask entries per voxel: the MIN reduce of CostVolumeV3 records (view, reference group,
@@ -1817,7 +1857,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
         const bool valid = hit.off >= 0;
         if (valid) {
           const unsigned fh = (unsigned)hit.key >> 16;
-          ring_rows[n] |= (1u << (fh & (WN::ROWS - 1))) | (1u << ((fh + 1u) & (WN::ROWS - 1)));
+          ring_rows[n] |= (1u << WN::ring_row(fh)) | (1u << WN::ring_row(fh + 1u));
         }
         bool in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
         chunk_out[n] = false;
@@ -1897,19 +1937,21 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
       }
       // The records of the NEXT depth are requested now, so that their LDS latency overlaps
       // this depth's arithmetic (jj is unrolled: the buffer index is a compile-time constant).
-      const int cb = jj & 1, nb = cb ^ 1;
+      // (a lean kernel reads the records of depth jj here, into the one set it keeps)
+      const int cb = kLean ? 0 : (jj & 1), nb = kLean ? 0 : (cb ^ 1);
+      constexpr int kAhead = kLean ? 0 : 1;
       if constexpr (LPP > 1) {
-        if (jj + 1 < LPP) {
+        if (kLean ? jj > 0 : jj + 1 < LPP) {
 #pragma unroll
           for (int n = 0; n < NV; ++n) {
-            rb_off[nb][n] = lds_at<int>(smem, p4, kOff + ((n * LPP + jj + 1) * PPW) * 4);
-            rb_wt[nb][n] = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj + 1) * PPW) * 16);
+            rb_off[nb][n] = lds_at<int>(smem, p4, kOff + ((n * LPP + jj + kAhead) * PPW) * 4);
+            rb_wt[nb][n] = lds_at<float4>(smem, p4 * 4u, kWts + ((n * LPP + jj + kAhead) * PPW) * 16);
             if constexpr (DG)
-              rb_dwt[nb][n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj + 1) * PPW) * 16);
+              rb_dwt[nb][n] = lds_at<float4>(smem, p4 * 4u, kDwt + ((n * LPP + jj + kAhead) * PPW) * 16);
             else
               rb_dwt[nb][n] = make_float4(0.f, 0.f, 0.f, 0.f);
           }
-          rb_scl[nb] = lds_at<float>(smem, p4, kScl + ((jj + 1) * PPW) * 4);
+          rb_scl[nb] = lds_at<float>(smem, p4, kScl + ((jj + kAhead) * PPW) * 4);
         }
       }
       const int *rec_off = rb_off[cb];
@@ -1993,8 +2035,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
               load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + (e1 + cb)), tap[n][2]);
               load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + e1), tap[n][3]);
               if (cur[n] >= 0)
-                window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
-                                     s_data + n * WN::SLOTS * WN::STRIDE, s_tags, t.lane, t.cl);
+                window_add<VEC, LPP, kLean>((unsigned)cell[n].x, cell[n].y, sg[n],
+                                            s_data + n * WN::SLOTS * WN::STRIDE, s_tags, t.lane, t.cl);
               cur[n] = off;
               if constexpr (LPP > 1)
                 cell[n] = lds_at<int2>(smem, p4 * 2u, kCell + ((n * LPP + jj) * PPW) * 8);
