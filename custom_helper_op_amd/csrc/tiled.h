@@ -1577,8 +1577,11 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 // four window taps of a pixel that fires alone added one after the other (12) -- 127 registers,
 // no scratch.  Those three cost 5 % at three waves per SIMD; with the 10 KB of LDS of the
 // six-row window the fourth wave gains 11 %.
+// Likewise the gradients of CostAggregate (both reduces: 137 -> 114 registers) and of
+// FeatureAggregate (149 -> 112).  Not the MIN / MAX gradients of the per-channel ops (their mask
+// rows keep them above 140) and not CostVolumeV3 (its two extra LDS rows per pixel are 2 KB).
 constexpr bool lean_backward(int nv, int lpp, int corr, int reduce) {
-  return nv == 1 && lpp == 8 && corr == 0 && reduce == 0;
+  return nv == 1 && lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4);
 }
 constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1) {
   return lean_backward(nv, lpp, corr, reduce)              ? 4
