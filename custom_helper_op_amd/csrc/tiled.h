@@ -1581,7 +1581,8 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 // FeatureAggregate (149 -> 112).  Not the MIN / MAX gradients of the per-channel ops (their mask
 // rows keep them above 140) and not CostVolumeV3 (its two extra LDS rows per pixel are 2 KB).
 constexpr bool lean_backward(int nv, int lpp, int corr, int reduce) {
-  return nv == 1 && lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4);
+  return nv == 1 && ((lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4)) ||
+                     (lpp == 4 && corr <= 1 && reduce == 0));
 }
 constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1) {
   return lean_backward(nv, lpp, corr, reduce)              ? 4
