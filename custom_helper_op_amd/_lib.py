@@ -20,6 +20,8 @@ SIGNATURES = {
     "chop_set_kernel_family": [_int],
     "chop_last_kernel_family": [],
     "chop_last_views_per_workgroup": [],
+    "chop_set_backward_window": [_int],
+    "chop_last_backward_window": [],
     "chop_cost_volume_bwd16_workspace_bytes": [_i64] * 7,
 }
 for _t in ("f32", "f64"):

@@ -18,6 +18,8 @@ thread_local std::string g_last_error = "";
 thread_local int g_kernel_family = 0;
 thread_local int g_last_family = 0;
 thread_local int g_last_views_per_workgroup = 0;
+thread_local int g_last_backward_window = 0;
+thread_local int g_backward_window = 0;  // 0: the launcher decides, 6, 8 (chop_set_backward_window)
 
 int fail(int code, const std::string &msg) {
   g_last_error = msg;
@@ -343,6 +345,8 @@ void *scratch_if_known() {
 }  // namespace
 
 void note_views_per_workgroup(int views) { g_last_views_per_workgroup = views; }
+int backward_window_mode() { return g_backward_window; }
+void note_backward_window(int rows) { g_last_backward_window = rows; }
 
 }  // namespace chop
 
@@ -373,6 +377,14 @@ int chop_set_kernel_family(int family) {
 }
 
 int chop_last_kernel_family(void) { return g_last_family; }
+
+int chop_last_backward_window(void) { return g_last_family == 2 ? g_last_backward_window : 0; }
+
+int chop_set_backward_window(int rows) {
+  const int prev = g_backward_window;
+  g_backward_window = rows == 6 || rows == 8 ? rows : 0;
+  return prev;
+}
 
 #define DIMS \
   Dims { B, H, W, C, D, N, srcH, srcW }

@@ -148,6 +148,11 @@ hipError_t launch_tiled_backward_wide(const Args<S> &a, hipStream_t stream);
 // The tiled backward launcher reports how many views a workgroup took in turn (api.hip keeps
 // it per host thread for chop_last_views_per_workgroup).
 void note_views_per_workgroup(int views);
+// The calling thread's choice between the two 32-channel tiled gradient kernels
+// (chop_set_backward_window): 0 the launcher decides, 6 slimmed, 8 wide.
+int backward_window_mode();
+// ... and which of the two the launcher took (0: a shape that has only one kernel)
+void note_backward_window(int rows);
 
 // Utility launches.
 hipError_t launch_fill_zero(void *ptr, size_t bytes, hipStream_t stream);

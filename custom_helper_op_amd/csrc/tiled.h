@@ -1192,18 +1192,19 @@ __attribute__((amdgpu_waves_per_eu(forward_min_waves(LPP, NV, CORR, REDUCE), 5))
 // holds exactly the texels [oy, oy+ROWS) x [ox, ox+COLS).  Because the slot of a texel
 // depends only on its coordinates, the four slots of a cell are computed once, by the lane
 // that reprojects the voxel, and travel with the record.
-template <int VEC, int LPP>
+template <int VEC, int LPP, bool SIX = false>
 struct Window {
   static constexpr int PPW = 64 / LPP;
   // twice the tile's height by twice its width, at least eight each way: room for the
   // samples' drift in either direction (8 x 8 against 4 x 16 for the 2 x 4 pixels of 32
   // channels: 357 -> 338 us on the MVSNet-stage workload)
   static constexpr int TH = tile_rows(PPW), TW = PPW / TH;
-  // Eight lanes per pixel (32 channels, 2 x 4 pixels): six rows instead of eight.  With a
-  // 6 KB window the workgroup's LDS is 10 KB, so that sixteen workgroups fit a CU (four waves
-  // per SIMD: see backward_waves); four rows measured 2 % slower than eight at equal
-  // occupancy, six sit between.  The ring index of a row is then a remainder, not a mask.
-  static constexpr int ROWS = LPP == 8 ? 6 : (2 * TH > 8 ? 2 * TH : 8);
+  // SIX (eight lanes per pixel, 32 channels, 2 x 4 pixels, kernels held to four waves per
+  // SIMD: see backward_waves): six rows instead of eight.  With a 6 KB window the workgroup's
+  // LDS is 10 KB, so that sixteen workgroups fit a CU; four rows measured 2 % slower than eight
+  // at equal occupancy, six sit between.  The ring index of a row is then a remainder, not a
+  // mask.
+  static constexpr int ROWS = SIX ? 6 : (2 * TH > 8 ? 2 * TH : 8);
   static constexpr int COLS = 2 * TW > 8 ? 2 * TW : 8;
   static constexpr int SLOTS = ROWS * COLS;
   static constexpr bool kPow2Rows = (ROWS & (ROWS - 1)) == 0;
@@ -1251,20 +1252,20 @@ constexpr int kClaimLanes = 8;
 // then the list of texels leaving a window, then the windows.  With one view per workgroup
 // the list shares the record space: a window only moves before the chunk's records are
 // written.
-template <int VEC, int LPP, int NV>
+template <int VEC, int LPP, int NV, bool SIX = false>
 constexpr int backward_record_words() {
-  using WN = Window<VEC, LPP>;
+  using WN = Window<VEC, LPP, SIX>;
   const int rec = LPP > 1 ? NV * 64 * 11 + 128 : 0;
   const int list = WN::SLOTS * 2;
   const int w = NV == 1 ? (rec > list ? rec : list) : rec + list;
   return (w + 3) / 4 * 4;
 }
-template <int VEC, int LPP, int NV>
+template <int VEC, int LPP, int NV, bool SIX = false>
 constexpr int backward_lds_words() {
-  using WN = Window<VEC, LPP>;
+  using WN = Window<VEC, LPP, SIX>;
   // records (or list), windows, one cell (4 texels x C) staged on its way to memory, and for
   // narrow pixels one claim word per window slot
-  return backward_record_words<VEC, LPP, NV>() + NV * WN::SLOTS * WN::STRIDE + 4 * WN::C +
+  return backward_record_words<VEC, LPP, NV, SIX>() + NV * WN::SLOTS * WN::STRIDE + 4 * WN::C +
          (LPP <= kClaimLanes ? WN::SLOTS : 0);
 }
 
@@ -1282,10 +1283,10 @@ __device__ __forceinline__ int wave_min(int v) {
 // Moves the window of one view to origin (ny, nx): every texel that falls outside the new
 // window is written out with dense global atomics (C consecutive floats per texel, 64/C
 // texels per instruction) and its slot is cleared.  Uniform control flow.
-template <int VEC, int LPP>
+template <int VEC, int LPP, bool SIX = false>
 __device__ __forceinline__ void window_move(int &oy, int &ox, int ny, int nx, float *data,
                                             int *list, float *gview, int srcW, int lane) {
-  using WN = Window<VEC, LPP>;
+  using WN = Window<VEC, LPP, SIX>;
   if (oy != WN::kNone) {
     wave_sync();  // the adds of the chunk before are complete and visible
     int count = 0;
@@ -1351,10 +1352,10 @@ __device__ __forceinline__ unsigned wave_or(unsigned v) {
 // set when a cell used ring row r; a short sweep over few hypotheses touches three or four
 // of the eight, and the untouched ones need neither their LDS reads nor their address
 // arithmetic).  All LDS reads of a row are issued together, then its atomics.
-template <int VEC, int LPP>
+template <int VEC, int LPP, bool SIX = false>
 __device__ __forceinline__ void window_flush_all(int oy, int ox, const float *data, float *gview,
                                                  int srcW, int lane, unsigned rows) {
-  using WN = Window<VEC, LPP>;
+  using WN = Window<VEC, LPP, SIX>;
   if (oy == WN::kNone) return;
   wave_sync();  // the last adds are complete and visible
   constexpr int C = WN::C;
@@ -1415,10 +1416,10 @@ __device__ __forceinline__ void window_flush_all(int oy, int ox, const float *da
 // from 429 to 400 us; against LDS atomics it halved the time of the 8-channel workloads.
 // 16 lanes per pixel (four pixels per wave): the pixels that fire in the same instruction
 // take turns, one pixel per round with its four taps in flight together.
-template <int VEC, int LPP, bool LEAN = false>
+template <int VEC, int LPP, bool LEAN = false, bool SIX = false>
 __device__ __forceinline__ void window_add(unsigned slots, int key, float (&v)[4][VEC],
                                            float *data, int *tags, int lane, int cl) {
-  using WN = Window<VEC, LPP>;
+  using WN = Window<VEC, LPP, SIX>;
   typedef float vecf __attribute__((ext_vector_type(VEC)));
   if (key < 0) {
     // the whole cell lies inside the window (the usual case)
@@ -1564,32 +1565,35 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 
 // Waves per SIMD the register budget is held to.  The kernel is latency-bound (its time
 // falls in proportion to the resident waves), so one view per workgroup at three waves
-// beats two views at two.
-// Four lanes per pixel (16 channels), gradient of a mean: the window of its 4 x 4 pixel tile is
-// 4 KB, which leaves LDS for sixteen workgroups per CU, and the kernel needs 130 registers left
-// alone; held to 128 it spills three to five of them and the fourth wave takes the f16 cascade
-// workload from 300 to 268 us.  (The MIN / MAX gradients, which stage mask rows as well, and
-// the ops with one upstream value per voxel would spill 15 to 35 registers: three waves.)
+// beats two views at two, and four waves beat three wherever registers and LDS allow them.
 // Eight lanes per pixel (32 channels), gradient of the mean squared difference: 161 registers
 // left alone.  Held to 128 it spills 80 bytes in the depth loop, so the kernel is slimmed
 // first (lean_backward): four upstream rows staged at a time instead of eight (16 registers),
 // the records of a depth read where the depth starts instead of one depth ahead (10), the
 // four window taps of a pixel that fires alone added one after the other (12) -- 127 registers,
 // no scratch.  Those three cost 5 % at three waves per SIMD; with the 10 KB of LDS of the
-// six-row window the fourth wave gains 11 %.
-// Likewise the gradients of CostAggregate (both reduces: 137 -> 114 registers) and of
-// FeatureAggregate (149 -> 112).  Not the MIN / MAX gradients of the per-channel ops (their mask
+// six-row window the fourth wave gains 11 % (MVSNet-stage backward 301 -> 277 us).
+// Likewise the gradients of CostAggregate (both reduces: 137 -> 117 registers) and of
+// FeatureAggregate (149 -> 119).  Not the MIN / MAX gradients of the per-channel ops (their mask
 // rows keep them above 140) and not CostVolumeV3 (its two extra LDS rows per pixel are 2 KB).
-constexpr bool lean_backward(int nv, int lpp, int corr, int reduce) {
-  return nv == 1 && ((lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4)) ||
-                     (lpp == 4 && corr <= 1 && reduce == 0));
+// Four lanes per pixel (16 channels), gradients of a mean: 130 registers left alone, 121 lean
+// (held to 128 without the slimming they spilled three to five); the window of the 4 x 4 pixel
+// tile is 4 KB.  Two lanes per pixel (8 channels): 119-125 lean -- unless the views of a tile
+// take turns in the workgroup (VLOOP), which costs 26 registers more: those kernels would
+// spill 44-68 bytes and stay at three waves, not slimmed (bf16 group-correlation backward 482 us
+// against 511 us lean with four).
+constexpr bool lean_backward(int nv, int lpp, int corr, int reduce, bool vloop = false,
+                             bool wide = false) {
+  return nv == 1 && !wide && ((lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4)) ||
+                     (lpp == 4 && corr <= 1 && reduce == 0) ||
+                     (lpp == 2 && corr <= 1 && reduce == 0 && !vloop));
 }
-constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1) {
-  return lean_backward(nv, lpp, corr, reduce)              ? 4
-         : nv == 1 && lpp == 4 && corr <= 1 && reduce == 0 ? 4
-         : nv == 1 && lpp <= 8                           ? 3
-         : nv <= 2                                       ? 2
-                                                         : 1;
+constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1, bool vloop = false,
+                             bool wide = false) {
+  return lean_backward(nv, lpp, corr, reduce, vloop, wide) ? 4
+         : nv == 1 && lpp <= 8                       ? 3
+         : nv <= 2                                   ? 2
+                                                     : 1;
 }
 
 // REDUCE: 0 gradient of the mean (mask = number of accepted views), 1 gradient of the
@@ -1605,11 +1609,20 @@ constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1) {
 // VLOOP: the workgroup's view group holds several views, which take turns (g.vper of them).
 // A compile-time flag: the loop around the kernel's body costs the wide instantiations
 // registers they do not have (the 32-channel kernel spills with it).
+// WIDE: the kernel as it is without the slimming of lean_backward: three waves per SIMD and, for
+// 32 channels, the 8 x 8 window.  For sweeps whose samples of consecutive hypotheses land many
+// texels apart (wide baselines, hypotheses close to the cameras) the two rows more are worth
+// more than the fourth wave: fewer cells stick out of the window and go to memory on their
+// own, and such launches are bound by those atomics, not by latency (six source views with
+// 15-degree rotations and depths from 0.5: 18.9 ms against 20.6 ms slimmed).  The launcher
+// decides (tiled_launch.inc).
 template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true,
-          bool PV = (CORR == 1), bool VLOOP = false>
-__global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void backward_kernel(const Args<S> a,
+          bool PV = (CORR == 1), bool VLOOP = false, bool WIDE = false>
+__global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, VLOOP, WIDE)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
-  using WN = Window<VEC, LPP>;
+  constexpr bool kLean = lean_backward(NV, LPP, CORR, REDUCE, VLOOP, WIDE);
+  constexpr bool kSix = kLean && LPP == 8;
+  using WN = Window<VEC, LPP, kSix>;
   constexpr int PPW = 64 / LPP;
   constexpr bool kWide = sizeof(S) == 2;  // gradients accumulate in fp32 images
   extern __shared__ __align__(16) unsigned char smem[];
@@ -1626,7 +1639,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
   const unsigned q4 = (unsigned)(t.cl * PPW + t.p) * 4u;       // writer: lane (p, j)
   int *s_list = NV == 1 ? reinterpret_cast<int *>(smem)
                         : reinterpret_cast<int *>(smem) + (LPP > 1 ? NV * 64 * 11 + 128 : 0);
-  float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV>();
+  float *s_data = reinterpret_cast<float *>(smem) + backward_record_words<VEC, LPP, NV, kSix>();
   float *s_stage = s_data + NV * WN::SLOTS * WN::STRIDE;
   int *s_tags = reinterpret_cast<int *>(s_stage + 4 * WN::C);  // narrow pixels: claim words
   static_assert(LPP > kClaimLanes || NV == 1, "one set of claim words: one view per workgroup");
@@ -1665,7 +1678,6 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
   const int gv = VEC / g.sub;
   const int d_lo = t.d_lo, d_hi = t.d_hi;
   // upstream-gradient rows fetched ahead; the MIN reduce stages the mask rows beside them
-  constexpr bool kLean = lean_backward(NV, LPP, CORR, REDUCE) && !VLOOP;
   constexpr int PFMAX = (REDUCE || kLean) ? 4 : 8;
   constexpr int PF = LPP < PFMAX ? LPP : PFMAX;
   constexpr bool kMaskRows = REDUCE == 1 && !kVoxelGrad;
@@ -1875,7 +1887,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
           const int ny = wave_min(my), nx = wave_min(mx);
           const int hy = -wave_min(-My) + 1, hx = -wave_min(-Mx) + 1;  // last row / column used
           const int sy = WN::ROWS - (hy - ny + 1), sx = WN::COLS - (hx - nx + 1);  // slack
-          window_move<VEC, LPP>(oy[n], ox[n], ny - (sy > 0 ? sy / 2 : 0),
+          window_move<VEC, LPP, kSix>(oy[n], ox[n], ny - (sy > 0 ? sy / 2 : 0),
                                 nx - (sx > 0 ? sx / 2 : 0), s_data + n * WN::SLOTS * WN::STRIDE,
                                 s_list, gview[n], srcW, t.lane);
           in_new = !valid || WN::inside(hit.key, oy[n], ox[n]);
@@ -2039,7 +2051,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
               load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + (e1 + cb)), tap[n][2]);
               load_vec<S, VEC, false>(reinterpret_cast<const S *>(vb + e1), tap[n][3]);
               if (cur[n] >= 0)
-                window_add<VEC, LPP, kLean>((unsigned)cell[n].x, cell[n].y, sg[n],
+                window_add<VEC, LPP, kLean, kSix>((unsigned)cell[n].x, cell[n].y, sg[n],
                                             s_data + n * WN::SLOTS * WN::STRIDE, s_tags, t.lane, t.cl);
               cur[n] = off;
               if constexpr (LPP > 1)
@@ -2140,13 +2152,13 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE)) void bac
       flush_cells_to_memory<VEC, LPP>(m, out, cell[n].y, sg[n], s_stage, gview[n], srcW, t.lane,
                                       t.cl);
     if (cur[n] >= 0 && !out)
-      window_add<VEC, LPP>((unsigned)cell[n].x, cell[n].y, sg[n],
+      window_add<VEC, LPP, false, kSix>((unsigned)cell[n].x, cell[n].y, sg[n],
                            s_data + n * WN::SLOTS * WN::STRIDE, s_tags, t.lane, t.cl);
   }
   wave_sync();
 #pragma unroll
   for (int n = 0; n < NV; ++n)
-    window_flush_all<VEC, LPP>(oy[n], ox[n], s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
+    window_flush_all<VEC, LPP, kSix>(oy[n], ox[n], s_data + n * WN::SLOTS * WN::STRIDE, gview[n], srcW,
                                t.lane, wave_or(ring_rows[n]));
   wave_sync();  // the next view clears the window
   }  // views of the group

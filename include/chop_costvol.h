@@ -426,6 +426,19 @@ int chop_last_kernel_family(void);
  * image, all views of a pixel tile in one workgroup); 0 if the last backward call did not run
  * the tiled kernels.  For the tests. */
 int chop_last_views_per_workgroup(void);
+/* No counterpart in the reference.  The tiled gradient kernels for 32 channels exist twice:
+ * slimmed to four wavefronts per SIMD with a scatter window of 6 x 8 texels, and at three
+ * wavefronts with 8 x 8.  The first is 8-11 % faster while the samples of consecutive depth
+ * hypotheses land close to each other (ordinary rigs), the second about 9 % where they do not
+ * (wide baselines with hypotheses close to the cameras).  The library cannot see the cameras
+ * from the host and picks the second for five or more source views; rows = 6 or 8 fixes the
+ * choice for subsequent calls from this thread, 0 returns it to the library.  Returns the
+ * previous value.  Results agree within the gradient tolerance either way. */
+int chop_set_backward_window(int rows);
+/* Which of the two the last tiled backward call of this thread ran: 6 or 8; 0 for a shape
+ * that has one kernel only, or if the last backward call did not run the tiled kernels.  For
+ * the tests. */
+int chop_last_backward_window(void);
 
 #ifdef __cplusplus
 }

@@ -9,7 +9,7 @@ import torch
 
 import custom_helper_op_amd as chop
 from custom_helper_op_amd import _lib
-from custom_helper_op_amd.configs import make_workload, quantise
+from custom_helper_op_amd.configs import make_workload, quantise, reference_test_case
 from gpu_util import TORCH_DTYPE, assert_backward_close, assert_forward_close, dev, host, rms
 
 pytestmark = pytest.mark.gpu
@@ -154,3 +154,59 @@ def test_feature_aggregate(oracle):
     _turns(3)
     for g, w in zip(got, want):
         assert_backward_close(host(g), w)
+
+
+@pytest.mark.parametrize("op", ["cost_volume", "cost_volume_f16", "cost_aggregate", "cost_aggregate_min",
+                                "feature_aggregate"])
+def test_both_32_channel_gradient_kernels(oracle, op):
+    """The 32-channel gradients exist slimmed (four waves per SIMD, 6 x 8 scatter window) and
+    wide (three waves, 8 x 8): both against the oracle, on a sweep long enough for the window
+    to move (and for cells to leave the smaller one), and the launcher's own choice by the
+    number of source views."""
+    lib = _lib.load()
+    B, H, W, C, D = 1, 24, 36, 32, 40
+    rng = np.random.default_rng(41)
+    for N, want_auto in ((2, 6), (5, 8)):
+        t = reference_test_case(2, B, N, H, W, C, D, np.float32, seed=70 + N)
+        args = tuple(t[k] for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts"))
+        if op.startswith("cost_volume"):
+            half = op.endswith("f16")
+            if half:
+                q = lambda x: x.astype(np.float16).astype(np.float32)
+                args = (q(args[0]), q(args[1])) + args[2:]
+            _, mask = oracle.cost_volume_fwd(*args, "MEAN")
+            cg = rng.normal(size=(B, H, W, D, C)).astype(np.float32)
+            if half:
+                cg = cg.astype(np.float16).astype(np.float32)
+            want = oracle.cost_volume_bwd(*args, cg, mask, "MEAN")
+            dt = torch.float16 if half else None
+            ins = [dev(args[0], dt), dev(args[1], dt)] + [dev(x) for x in args[2:]]
+            run = lambda: chop.cost_volume_grad(*ins, dev(cg, dt), dev(mask), "MEAN")
+            rtol = 1e-2 if half else 1e-4
+        elif op.startswith("cost_aggregate"):
+            reduce = "MIN" if op.endswith("min") else "MEAN"
+            _, mask = oracle.cost_aggregate_fwd(*args, reduce)
+            cg = rng.normal(size=(B, H, W, D)).astype(np.float32)
+            want = oracle.cost_aggregate_bwd(*args, cg, mask, reduce)
+            ins = [dev(x) for x in args]
+            run = lambda: chop.cost_aggregate_grad(*ins, dev(cg), dev(mask), reduce)
+            rtol = 1e-4
+        else:
+            fargs = args[1:]
+            _, mask = oracle.feature_aggregate_fwd(*fargs)
+            cg = rng.normal(size=(B, H, W, D, N, C)).astype(np.float32)
+            want = oracle.feature_aggregate_bwd(*fargs, cg, mask)
+            ins = [dev(x) for x in fargs]
+            run = lambda: chop.feature_aggregate_grad(*ins, dev(cg), dev(mask))
+            rtol = 1e-4
+        for rows in (6, 8, 0):
+            print("\n[case] %s N=%d window %d" % (op, N, rows), flush=True)
+            lib.chop_set_backward_window(rows)
+            try:
+                got = run()
+                assert lib.chop_last_kernel_family() == 2
+                assert lib.chop_last_backward_window() == (rows if rows else want_auto)
+            finally:
+                lib.chop_set_backward_window(0)
+            for g, w in zip(got, want):
+                assert_backward_close(host(g), w, rtol=rtol)
