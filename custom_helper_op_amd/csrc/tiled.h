@@ -1578,15 +1578,17 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 // rows keep them above 140) and not CostVolumeV3 (its two extra LDS rows per pixel are 2 KB).
 // Four lanes per pixel (16 channels), gradients of a mean: 130 registers left alone, 121 lean
 // (held to 128 without the slimming they spilled three to five); the window of the 4 x 4 pixel
-// tile is 4 KB.  Two lanes per pixel (8 channels): 119-125 lean -- unless the views of a tile
-// take turns in the workgroup (VLOOP), which costs 26 registers more: those kernels would
-// spill 44-68 bytes and stay at three waves, not slimmed (bf16 group-correlation backward 482 us
-// against 511 us lean with four).
+// tile is 4 KB.  Two lanes per pixel (8 channels): 119-125 lean, and 122-128 where the views of
+// a tile take turns in the workgroup (VLOOP) -- once the compiler is kept from carrying two
+// dozen lane-only values through the view loop (see the barrier at the head of that loop;
+// with them the kernels spilled 44-68 bytes around the depth loop and four waves were slower
+// than three).  Up to 32 bytes of scratch remain in two of those instantiations, outside the
+// depth loop: bf16 group-correlation backward 479 -> 462 us cold, 447 -> 417 us warm.
 constexpr bool lean_backward(int nv, int lpp, int corr, int reduce, bool vloop = false,
                              bool wide = false) {
   return nv == 1 && !wide && ((lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4)) ||
                      (lpp == 4 && corr <= 1 && reduce == 0) ||
-                     (lpp == 2 && corr <= 1 && reduce == 0 && !vloop));
+                     (lpp == 2 && corr <= 1 && reduce == 0));
 }
 constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1, bool vloop = false,
                              bool wide = false) {
@@ -1696,6 +1698,13 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, VLOOP, WI
   const int group_views = VLOOP ? min(g.vper > NV ? g.vper : NV, N - first_view) : NV;
   for (int vi = 0; vi < group_views; vi += NV) {
   t.view0 = first_view + vi;
+  if constexpr (VLOOP) {
+    // The lane index as a value the compiler cannot see through: without this it computes
+    // everything that depends only on the lane (slot and row arithmetic of the window moves
+    // and flushes) once in front of the view loop and keeps it in registers through all
+    // views -- two dozen registers the depth loop needs.
+    asm volatile("" : "+v"(t.lane), "+v"(t.cl), "+v"(t.p), "+v"(t.pix), "+v"(t.h), "+v"(t.w));
+  }
   for (int k = t.lane * 4; k < NV * WN::SLOTS * WN::STRIDE; k += 256)
     *reinterpret_cast<float4 *>(s_data + k) = make_float4(0.f, 0.f, 0.f, 0.f);
   Cameras<NV> cam;
