@@ -615,6 +615,22 @@ def test_large_batch_stress_full_size():
     for a1, a2 in zip(g1, g2):
         scale = float(a1.abs().max())
         assert float((a2 - 2 * a1).abs().max()) <= 2e-4 * scale
+    # Six source views: the launcher took the wide form of the 32-channel kernel (three waves
+    # per SIMD, 8 x 8 scatter window).  The slimmed form (four waves, 6 x 8 window), in which
+    # far more of this workload's cells stick out of the window and go to memory on their own,
+    # must agree with it.
+    lib = _lib.load()
+    assert lib.chop_last_backward_window() == 8
+    lib.chop_set_backward_window(6)
+    try:
+        g3 = chop.cost_volume_grad(*ins, cg, mask)
+        assert lib.chop_last_backward_window() == 6
+    finally:
+        lib.chop_set_backward_window(0)
+    for a2, a3 in zip(g2, g3):
+        scale = float(a2.abs().max())
+        assert float((a3 - a2).abs().max()) <= 2e-4 * scale
+    assert_backward_close(host(g3[0][b:b + 1, :r1]) / 2, want[0], what="ref_grad band, slimmed kernel")
 
 
 def test_volume_above_two_to_the_31_elements():
