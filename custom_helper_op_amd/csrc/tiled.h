@@ -52,6 +52,7 @@ struct Geometry {
   int vper;                // views per group
   int seg;                 // depths per segment, multiple of LPP
   int64_t total_units;     // B * tiles_per_image * nseg * ngroups
+  unsigned units_per_seg;  // B * tiles_per_image * ngroups
   int64_t units_per_xcd;   // ceil(total_units / 8)
   int xcd_shift;           // log2 of the units dealt to one XCD at a time; -1: one band per XCD
   int64_t grid;            // workgroups to launch
@@ -320,11 +321,26 @@ __device__ __forceinline__ bool locate_tile(const Args<S> &a, const Geometry &g,
   if (unit >= (unsigned)g.total_units) return false;
   // the groups of one (tile, segment) are neighbours in launch order: they stream the same
   // upstream-gradient rows at about the same time, through the same L2
-  const unsigned per_tile = (unsigned)(g.nseg * g.ngroups);
-  const unsigned tile = unit / per_tile;
-  const int rem = (int)(unit - tile * per_tile);
-  const int segi = rem / g.ngroups;
-  t.view0 = (rem - segi * g.ngroups) * g.vper;
+  unsigned tile;
+  int segi;
+  if (g.xcd_shift >= 0) {
+    // Backward: the depth segments one after the other, all tiles of the first segment first.
+    // The workgroups of a launch differ in length, and what the chip does while the last ones
+    // finish is lost; the segment of the nearest hypotheses (most cell changes per depth) is
+    // the longest, so it goes first and the launch ends on the shortest workgroups
+    // (MVSNet-stage backward -2.5 %; the far segment first: +0.5 %).
+    const unsigned sraw = unit / g.units_per_seg;
+    const unsigned rem = unit - sraw * g.units_per_seg;
+    segi = (int)sraw;
+    tile = rem / (unsigned)g.ngroups;
+    t.view0 = (int)(rem - tile * (unsigned)g.ngroups) * g.vper;
+  } else {
+    const unsigned per_tile = (unsigned)(g.nseg * g.ngroups);
+    tile = unit / per_tile;
+    const int rem = (int)(unit - tile * per_tile);
+    segi = rem / g.ngroups;
+    t.view0 = (rem - segi * g.ngroups) * g.vper;
+  }
   t.d_lo = segi * g.seg;
   t.d_hi = min((int)a.D, t.d_lo + g.seg);
   t.b = (int)(tile / (unsigned)g.tiles_per_image);
@@ -2233,6 +2249,7 @@ inline Geometry make_geometry(int64_t B, int64_t H, int64_t W, int64_t D, int su
   g.seg = ((per_seg + LPP - 1) / LPP) * LPP;
   g.nseg = (int)((D + g.seg - 1) / g.seg);
   g.total_units = tiles * g.nseg * g.ngroups;
+  g.units_per_seg = (unsigned)(tiles * g.ngroups);
   // backward: runs of 32 units (the view groups of a tile are neighbours and mostly share
   // a run, hence an L2)
   g.xcd_shift = vper > 0 ? 5 : -1;
