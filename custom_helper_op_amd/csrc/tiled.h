@@ -1600,15 +1600,13 @@ __device__ __forceinline__ void flush_cells_to_memory(unsigned long long m, bool
 // with them the kernels spilled 44-68 bytes around the depth loop and four waves were slower
 // than three).  Up to 32 bytes of scratch remain in two of those instantiations, outside the
 // depth loop: bf16 group-correlation backward 479 -> 462 us cold, 447 -> 417 us warm.
-constexpr bool lean_backward(int nv, int lpp, int corr, int reduce, bool vloop = false,
-                             bool wide = false) {
+constexpr bool lean_backward(int nv, int lpp, int corr, int reduce, bool wide = false) {
   return nv == 1 && !wide && ((lpp == 8 && ((corr == 0 && reduce == 0) || corr == 2 || corr == 4)) ||
                      (lpp == 4 && corr <= 1 && reduce == 0) ||
                      (lpp == 2 && corr <= 1 && reduce == 0));
 }
-constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1, bool vloop = false,
-                             bool wide = false) {
-  return lean_backward(nv, lpp, corr, reduce, vloop, wide) ? 4
+constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1, bool wide = false) {
+  return lean_backward(nv, lpp, corr, reduce, wide) ? 4
          : nv == 1 && lpp <= 8                       ? 3
          : nv <= 2                                   ? 2
                                                      : 1;
@@ -1636,9 +1634,9 @@ constexpr int backward_waves(int nv, int lpp, int corr = 0, int reduce = 1, bool
 // decides (tiled_launch.inc).
 template <typename S, int VEC, int LPP, int NV, int CORR, int REDUCE = 0, bool DG = true,
           bool PV = (CORR == 1), bool VLOOP = false, bool WIDE = false>
-__global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, VLOOP, WIDE)) void backward_kernel(const Args<S> a,
+__global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, WIDE)) void backward_kernel(const Args<S> a,
                                                                           const Geometry g) {
-  constexpr bool kLean = lean_backward(NV, LPP, CORR, REDUCE, VLOOP, WIDE);
+  constexpr bool kLean = lean_backward(NV, LPP, CORR, REDUCE, WIDE);
   constexpr bool kSix = kLean && LPP == 8;
   using WN = Window<VEC, LPP, kSix>;
   constexpr int PPW = 64 / LPP;
