@@ -321,7 +321,8 @@ def other_configs(torch, lib, make_workload, skip_index, scratch):
             "voxels": wl.voxels, "forward_ms": fwd_ms, "backward_ms": bwd_ms,
             "forward_frac": frac(fwd_b, fwd_ms), "backward_frac": frac(bwd_b, bwd_ms),
             "fwd_bwd_frac": frac(fwd_b + bwd_b, fwd_ms + bwd_ms),
-            "voxels_per_s": wl.voxels / ((fwd_ms + bwd_ms) * 1e-3)}
+            "voxels_per_s": wl.voxels / ((fwd_ms + bwd_ms) * 1e-3),
+            "backward_window_rows": lib.chop_last_backward_window()}
         del r
         torch.cuda.empty_cache()
     return out
@@ -352,6 +353,10 @@ def main():
     ap.add_argument("--kernel-family", choices=["auto", "general", "strip"], default="auto",
                     help="force the one-thread-per-element or the strip kernels instead of the "
                          "library's own choice")
+    ap.add_argument("--backward-window", type=int, choices=[0, 6, 8], default=0,
+                    help="fix the choice between the two 32-channel gradient kernels (6: four waves "
+                         "per SIMD, 6 x 8 scatter window; 8: three waves, 8 x 8) instead of the "
+                         "library's own (0)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference "
                          "that HBM traffic counters of a profiler run are scaled by")
@@ -369,6 +374,7 @@ def main():
     from custom_helper_op_amd.configs import make_workload
     lib = _lib.load()
     lib.chop_set_kernel_family({"auto": 0, "general": 1, "strip": 2}[a.kernel_family])
+    lib.chop_set_backward_window(a.backward_window)
     wl = make_workload(a.workload, with_cost_grad=False)
     wl.reduce_method = a.reduce
     if a.float64 or a.channels:
@@ -398,6 +404,8 @@ def main():
     served = [lib.chop_last_kernel_family()]
     r.backward()
     served.append(lib.chop_last_kernel_family())
+    # which of the two 32-channel gradient kernels the launcher took (0: the shape has one only)
+    backward_window = lib.chop_last_backward_window()
     served = "/".join({1: "general", 2: "tiled", 3: "strip"}.get(c, str(c)) for c in served)
     for _ in range(a.warmup):
         r.forward()
@@ -489,7 +497,7 @@ def main():
             wl.B, wl.N, wl.H, wl.W,
             wl.C, wl.D, " G%d" % wl.groups if wl.op in ("v2", "v3") else "", wl.storage),
             "voxels": wl.voxels, "reduce_method": wl.reduce_method, "half_centor": True,
-            "kernels": served},
+            "kernels": served, "backward_window_rows": backward_window},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "timing": "HIP events on the launch stream, caches overwritten before each call, median",
