@@ -8,8 +8,11 @@ synthetic input that is already resident in HBM.  Prints one JSON line.
 
 ``value`` and ``ms_per_step`` are wall-clock over exactly K back-to-back steps.  The
 ``roofline`` object is per call: HIP-event times of the dominant kernel's entry point with
-L2 and the memory-side cache overwritten before every call (cold), the back-to-back (warm)
-times beside them, and the rate a plain fill / copy reaches on this box in the same run.
+nothing of the workload in L2 or the memory-side cache (cold: a 1 GiB buffer is overwritten
+and then read before every call, so the caches hold clean lines of foreign data), the times
+right after the overwrite alone (every line dirty: the call also waits for the write-back of
+another kernel's output) and the back-to-back (warm) times beside them, and the rate a plain
+fill / copy reaches on this box in the same run.
 ``configs`` holds the cold forward / backward times of all five benchmark configurations.
 
 The default run is the headline configuration (workload 2, MEAN).  ``--reduce MIN``,
@@ -243,21 +246,30 @@ def cpu_baseline(wl, budget_s=12.0):
                       "cost and mask pre-allocated" % (wl.name, rows, wl.H, wl.D, len(times))}
 
 
-def timed_passes(torch, r, passes, scratch):
+def timed_passes(torch, r, passes, scratch, read_back=True):
     """`passes` forward + backward calls with HIP events on the launch stream around each
     call.  With `scratch` (a 1 GiB buffer) every call is preceded by an overwrite of it, so
-    that L2 and the memory-side cache hold nothing of the workload: cold-cache times."""
+    that L2 and the memory-side cache hold nothing of the workload: cold-cache times.  With
+    `read_back` the buffer is then read once, which leaves the caches full of clean lines;
+    without, every line is dirty and the first misses of the call push out another kernel's
+    output (kernels whose loads allocate in the caches then wait for those write-backs)."""
     ev = lambda: torch.cuda.Event(enable_timing=True)
     marks = []
+    sink = torch.zeros((), dtype=torch.float32, device="cuda:0") if scratch is not None else None
+
+    def flush(value):
+        if scratch is not None:
+            scratch.fill_(value)
+            if read_back:
+                sink.add_(scratch.sum())
+
     for _ in range(passes):
         e0, e1, e2, e3 = ev(), ev(), ev(), ev()
-        if scratch is not None:
-            scratch.fill_(1.0)
+        flush(1.0)
         e0.record()
         r.forward()
         e1.record()
-        if scratch is not None:
-            scratch.fill_(2.0)
+        flush(2.0)
         e2.record()
         r.backward()
         e3.record()
@@ -312,6 +324,7 @@ def other_configs(torch, lib, make_workload, skip_index, scratch):
             r.backward()
         torch.cuda.synchronize()
         fwd_ms, bwd_ms = timed_passes(torch, r, 9, scratch)
+        dirty_fwd, dirty_bwd = timed_passes(torch, r, 9, scratch, read_back=False)
         fwd_b, bwd_b = wl.algorithmic_bytes()
         frac = lambda b, ms: b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         out[wl.name] = {
@@ -322,6 +335,7 @@ def other_configs(torch, lib, make_workload, skip_index, scratch):
             "forward_frac": frac(fwd_b, fwd_ms), "backward_frac": frac(bwd_b, bwd_ms),
             "fwd_bwd_frac": frac(fwd_b + bwd_b, fwd_ms + bwd_ms),
             "voxels_per_s": wl.voxels / ((fwd_ms + bwd_ms) * 1e-3),
+            "after_overwrite_ms": {"forward": dirty_fwd, "backward": dirty_bwd},
             "backward_window_rows": lib.chop_last_backward_window()}
         del r
         torch.cuda.empty_cache()
@@ -455,11 +469,14 @@ def main():
         print("bench.py: graph replay skipped: %s" % e, file=sys.stderr)
     finally:
         r.stream = eager_stream
-    # per-call times, outside the timed region: warm (back to back, as above) and cold (the
-    # caches overwritten before every call); the roofline line is the cold one
+    # per-call times, outside the timed region: warm (back to back, as above), cold (a foreign
+    # buffer overwritten and read before every call) and right after the overwrite alone; the
+    # roofline line is the cold one
     warm_fwd, warm_bwd = timed_passes(torch, r, max(a.steps, 5), None)
     scratch = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0")
     fwd_ms, bwd_ms = timed_passes(torch, r, max(a.steps, 5), scratch)
+    dirty_fwd, dirty_bwd = timed_passes(torch, r, max(a.steps, 5), scratch, read_back=False)
+    dirty_ms = dirty_bwd if bwd_ms >= fwd_ms else dirty_fwd
     fwd_b, bwd_b = wl.algorithmic_bytes()
     dominant = "backward" if bwd_ms >= fwd_ms else "forward"
     d_ms, d_b = (bwd_ms, bwd_b) if dominant == "backward" else (fwd_ms, fwd_b)
@@ -500,7 +517,8 @@ def main():
             "kernels": served, "backward_window_rows": backward_window},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "timing": "HIP events on the launch stream, caches overwritten before each call, median",
+                     "timing": "HIP events on the launch stream, a foreign 1 GiB buffer overwritten and then "
+                               "read before each call (caches cold and clean), median",
                      "traffic": traffic, "traffic_source": traffic_source,
                      "traffic_stale": traffic_stale,
                      "algorithmic_bytes": {"forward": fwd_b, "backward": bwd_b},
@@ -510,6 +528,12 @@ def main():
                               "frac": d_b / (w_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                               "fwd_bwd_frac": (fwd_b + bwd_b) / ((warm_fwd + warm_bwd) * 1e-3) / 1e9
                                               / HBM_PEAK_GBS},
+                     "after_overwrite": {"ms": {"forward": dirty_fwd, "backward": dirty_bwd},
+                                         "frac": d_b / (dirty_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                         "fwd_bwd_frac": (fwd_b + bwd_b) / ((dirty_fwd + dirty_bwd) * 1e-3)
+                                                         / 1e9 / HBM_PEAK_GBS,
+                                         "note": "the 1 GiB buffer overwritten and not read: every cache "
+                                                 "line dirty with foreign data when the call starts"},
                      "measured_stream_GBs": stream,
                      "measured_stream": {**rates, "used": "copy" if dominant == "backward" else "fill"},
                      "frac_of_measured_stream": achieved / stream},

@@ -1807,10 +1807,7 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, WIDE)) vo
 #pragma unroll
           for (int jj = 0; jj < PF; ++jj) {
             const int d = min(first + jj, d_hi - 1);
-            // (streamed past the caches only where a pixel's row covers whole lines: narrower
-            // rows share their line with the neighbouring depths' rows, which later loads want)
-            load_vec<S, CNT, whole_lines(CNT * LPP, (int)sizeof(S))>(
-                cg_lane + (int64_t)d * cg_step, reinterpret_cast<float *>(cgw[jj]));
+            load_vec<S, CNT, false>(cg_lane + (int64_t)d * cg_step, reinterpret_cast<float *>(cgw[jj]));
           }
         };
         if (g.sub == 1) group_rows(std::integral_constant<int, VEC>());
@@ -1822,7 +1819,16 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, WIDE)) vo
       for (int jj = 0; jj < PF; ++jj) {
         const int d = min(first + jj, d_hi - 1);
         const S *src_cg = cg_lane + (int64_t)d * cg_step;
-        if constexpr (CORR == 0 || CORR == 4)
+        // (upstream rows and mask rows are read again by the workgroups of the tile's other
+        // views, which run next to this one on the same XCD: through the caches.  Streamed
+        // past them, the second view of the MVSNet-stage workload fetched 2 x 60 MB more from
+        // memory and the launch took 10 us longer in every cache state but one -- all lines
+        // dirty with another kernel's output, which a load that allocates has to push out
+        // first.  Each view of FeatureAggregate has rows of its own: streamed where they cover
+        // whole lines.)
+        if constexpr (CORR == 0)
+          load_raw<S, VEC, false>(src_cg, cgw[jj]);
+        if constexpr (CORR == 4)
           load_raw<S, VEC, whole_lines(VEC * LPP, (int)sizeof(S))>(src_cg, cgw[jj]);
         if constexpr (kMaskRows) {
           const int32_t *m = mask_lane + (int64_t)d * OC;
@@ -1830,15 +1836,15 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, WIDE)) vo
           if (cntv == 4) {
             typedef int i32x4 __attribute__((ext_vector_type(4)));
             const i32x4 *q = reinterpret_cast<const i32x4 *>(m);
-            const i32x4 v = whole_lines(4 * LPP, 4) ? __builtin_nontemporal_load(q) : *q;
+            const i32x4 v = *q;
             mrow[jj][0] = v[0], mrow[jj][1] = v[1], mrow[jj][2] = v[2], mrow[jj][3] = v[3];
           } else if (cntv == 2) {
             typedef int i32x2 __attribute__((ext_vector_type(2)));
             const i32x2 *q = reinterpret_cast<const i32x2 *>(m);
-            const i32x2 v = whole_lines(2 * LPP, 4) ? __builtin_nontemporal_load(q) : *q;
+            const i32x2 v = *q;
             mrow[jj][0] = v[0], mrow[jj][1] = v[1];
           } else {
-            mrow[jj][0] = whole_lines(LPP, 4) ? __builtin_nontemporal_load(m) : *m;
+            mrow[jj][0] = *m;
           }
         }
       }
