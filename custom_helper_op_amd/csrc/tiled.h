@@ -1788,12 +1788,12 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, WIDE)) vo
     float4 r_wts[NV], r_dwt[NV];
     bool chunk_out[NV];  // some cell of this chunk (or the open one) sticks out of the window
     // Issue the loads of this chunk's cost_grad rows now, unconditionally, so that the
-    // reprojection below overlaps their latency.  Streaming loads, although the workgroups of
-    // a tile's views read the same rows and only about half of the later reads find them in
-    // L2.  Cached loads for every view but the last fetch 676 instead of 830 MB on the
-    // two-view benchmark tensors and save 2 % with warm caches, but the rows they leave
-    // behind in L2 and the memory-side cache cost the next forward launch 5 us, and after
-    // other work has filled the caches with dirty lines they are 3 % slower than streaming.
+    // reprojection below overlaps their latency.  Through the caches: the workgroups of a
+    // tile's views read the same rows (streamed, only about a third of the later reads found
+    // them in L2).  At three waves per SIMD that was worth 2 % and cost the next forward launch
+    // 5 us; at four waves it is worth 4 %, the forward launch does not notice, and 13 % less
+    // is fetched.  One cache state is slower this way (by 4 %): every line dirty with another
+    // kernel's output, which a load that allocates has to push out first.
     // (whole rows are kept as loaded and widened to float where a depth uses them; group
     // rows, whose width is a run-time value, are widened here and kept as float bits)
     uint32_t cgw[kVoxelGrad ? 1 : PF][(CORR == 0 || CORR == 4) ? raw_words<S, VEC>() : VEC];
@@ -1819,13 +1819,8 @@ __global__ __launch_bounds__(64, backward_waves(NV, LPP, CORR, REDUCE, WIDE)) vo
       for (int jj = 0; jj < PF; ++jj) {
         const int d = min(first + jj, d_hi - 1);
         const S *src_cg = cg_lane + (int64_t)d * cg_step;
-        // (upstream rows and mask rows are read again by the workgroups of the tile's other
-        // views, which run next to this one on the same XCD: through the caches.  Streamed
-        // past them, the second view of the MVSNet-stage workload fetched 2 x 60 MB more from
-        // memory and the launch took 10 us longer in every cache state but one -- all lines
-        // dirty with another kernel's output, which a load that allocates has to push out
-        // first.  Each view of FeatureAggregate has rows of its own: streamed where they cover
-        // whole lines.)
+        // (each view of FeatureAggregate has rows of its own: streamed where they cover whole
+        // lines)
         if constexpr (CORR == 0)
           load_raw<S, VEC, false>(src_cg, cgw[jj]);
         if constexpr (CORR == 4)
