@@ -64,6 +64,11 @@ __device__ __forceinline__ double quick_recip(double x) {
   return __builtin_fma(__builtin_fma(-x, r, 1.0), r, r);
 }
 
+// a * b + c in one rounding: the backward's arithmetic (gradients are compared at 1e-4; with
+// contraction off for the whole library a plain a * b + c is two instructions)
+__device__ __forceinline__ float mad(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double mad(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
 // Sum over the 2^shift consecutive lanes of a pixel, left in every one of them.
 template <typename R>
 __device__ __forceinline__ R pixel_sum(R v, int shift) {
@@ -344,8 +349,17 @@ __global__ __launch_bounds__(64) void strip_forward_kernel(const Args<S> a, cons
 // ------------------------------------------------------------------------------------------
 // Backward
 // ------------------------------------------------------------------------------------------
-template <typename S, int CORR, int REDUCE>
-__global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, const StripGeom g) {
+// W4: compiled for four waves per SIMD.  In double the kernel needs 128-168 registers as
+// written; held to 128 (20-56 bytes of scratch per lane for most terms and reduces, up to 160
+// for the group correlation's maximum) it runs four waves instead of three wherever LDS lets
+// it, which is worth 12-22 % with wide pixels (see strip_geometry).  The gradients of a mean
+// take that form always (130 registers as written; narrow pixels gain 4-6 %), those of a
+// minimum / maximum only with wide pixels (3 channels in double: 6 % slower with the scratch
+// and nothing to gain, LDS holds such launches to ten workgroups per compute unit).  Float
+// and 16-bit storage stay below 128 registers by themselves.
+
+template <typename S, int CORR, int REDUCE, bool W4 = false>
+__global__ __launch_bounds__(64, W4 ? 4 : 1) void strip_backward_kernel(const Args<S> a, const StripGeom g) {
   using R = typename Storage<S>::Real;
   using Acc = typename std::conditional<sizeof(S) == 2, float, S>::type;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -369,7 +383,11 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
   const int oc = CORR == 1 ? (ch_ok ? cl / sub : 0) : (AGG || PAIR) ? 0 : (ch_ok ? cl : 0);
   const R ref_c = ch_ok && !FEAT ? Storage<S>::load(a.ref + px.pix * C + cl) : R(0);
   const R base = a.depth_grid ? R(0) : a.base_plane[px.pix];
-  const bool per_voxel = a.depth_grid != nullptr, want_depth = a.depth_grad != nullptr;
+  // per-voxel hypotheses: always for the group correlation, never for the ops over a base
+  // plane; the squared difference has them through the 16-bit entry points only (known at
+  // compile time wherever possible: the per-voxel sums of a chunk are 16 registers in double)
+  const bool per_voxel = CORR == 1 || (CORR == 0 && sizeof(S) == 2 && a.depth_grid != nullptr);
+  const bool want_depth = a.depth_grad != nullptr;
   const int64_t row_step = (int64_t)srcW * C;
   // fields: the four weights, dh, dw, the two depth-chain factors, 1 / view count
   // (CostAggregate: 1 / (view count * channels), or 1 / channels for the MIN reduce)
@@ -573,7 +591,10 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
             if (win[jj] != n) continue;  // another view won (:553)
           const R k00 = rec.at(0, ridx + jj), k01 = rec.at(1, ridx + jj), k11 = rec.at(2, ridx + jj),
                   k10 = rec.at(3, ridx + jj);
-          const R smp = k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10;
+          // (CostVolumeV3 compares dot products of these samples with the forward pass's: there
+          // the literal, separately rounded form)
+          const R smp = PAIR ? k00 * v00 + k01 * v01 + k11 * v11 + k10 * v10
+                             : mad(k10, v10, mad(k11, v11, mad(k01, v01, k00 * v00)));
           const R cg = cgv[jj];
           // CostVolumeV3 (cost_volume_kernels_gpu_v3.cu.cc:447-520, :593-640): the pair (reference
           // group gi, source group gs) this view contributed -- searched again for the mean (source
@@ -621,7 +642,7 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
             gv = cg;  // feature_aggregate_kernels_gpu.cu.cc:307-311
           } else if constexpr (PAIR) {
             const R scl = REDUCE == 0 ? cg * inv : cg;  // :426, :621
-            if (my_group == gi) racc += scl * s_smp[p * lpp + gs * sub + my_k];
+            if (my_group == gi) racc = mad(scl, s_smp[p * lpp + gs * sub + my_k], racc);
             if (my_group != gs) continue;  // only the winning source group receives a gradient
             gv = scl * s_ref[p * lpp + gi * sub + my_k];
           } else if (CORR != 1) {
@@ -630,18 +651,18 @@ __global__ __launch_bounds__(64) void strip_backward_kernel(const Args<S> a, con
             racc += -gv;
           } else {
             gv = REDUCE == 0 ? cg * inv : cg;  // v2 :461, :583
-            racc += gv * smp;
+            racc = mad(gv, smp, racc);
             gv = gv * ref_c;
           }
-          g00 += gv * k00;
-          g01 += gv * k01;
-          g11 += gv * k11;
-          g10 += gv * k10;
+          g00 = mad(gv, k00, g00);
+          g01 = mad(gv, k01, g01);
+          g11 = mad(gv, k11, g11);
+          g10 = mad(gv, k10, g10);
           if (want_depth) {
             const R t1 = v11 - v10 - v01 + v00;
-            const R h_grad = gv * (t1 * rec.at(5, ridx + jj) + v10 - v00);
-            const R w_grad = gv * (t1 * rec.at(4, ridx + jj) + v01 - v00);
-            const R dl = rec.at(6, ridx + jj) * h_grad + rec.at(7, ridx + jj) * w_grad;
+            const R h_grad = gv * mad(t1, rec.at(5, ridx + jj), v10 - v00);
+            const R w_grad = gv * mad(t1, rec.at(4, ridx + jj), v01 - v00);
+            const R dl = mad(rec.at(6, ridx + jj), h_grad, rec.at(7, ridx + jj) * w_grad);
             if (per_voxel)
               dvox[jj] += dl;
             else
@@ -747,6 +768,12 @@ StripGeom strip_geometry(const Args<S> &a) {
             a.B * a.N * a.srcH * a.srcW < (int64_t)1 << 31 && a.srcH < 32768 && a.srcW < 65536 &&
             rec_bytes + (g.carry ? strip_run_bytes<S>(a.N) : 0) + strip_cache_bytes<R>(a.N, lpp) <=
                 kMaxDynamicLds;
+  // With the cache a run that ends with its chunk costs a read-add-write in LDS, not atomics:
+  // the runs are not carried then, and without their 5 KiB (two views) sixteen workgroups fit a
+  // compute unit instead of thirteen -- the fourth wave per SIMD the kernel is compiled for.
+  // Float64, 32 channels, two views: 995 -> 866 us for the mean's gradient, 986 -> 950 us for
+  // the minimum's, 984 -> 896 us FeatureAggregate, 2810 -> 2233 us CostVolumeV3.
+  if (g.cache) g.carry = 0;
   return g;
 }
 
@@ -761,6 +788,11 @@ bool strip_supported(const Args<S> &a) {
   if (a.corr == GROUP_CORRELATION && (a.groups < 1 || a.C % a.groups != 0)) return false;
   if (a.srcH < 2 || a.srcW < 2) return false;                   // no sample can be accepted
   if (a.srcH * a.srcW * a.C >= (int64_t)1 << 31) return false;  // 32-bit offsets inside a view
+  // per-voxel hypotheses belong to the group correlation (always) and to the squared difference
+  // in 16-bit storage (by choice): the backward kernel knows this at compile time
+  const bool grid = a.depth_grid != nullptr;
+  if (a.corr == GROUP_CORRELATION ? !grid : grid && !(a.corr == SQUARED_DIFFERENCE && sizeof(S) == 2))
+    return false;
   const StripGeom g = strip_geometry(a);
   return g.tiles * g.nseg < (int64_t)1 << 31;
 }
@@ -836,31 +868,31 @@ hipError_t launch_strip_backward(const Args<S> &a, hipStream_t stream) {
                       (g.carry ? strip_run_bytes<S>(a.N) : 0) +
                       (g.cache ? strip_cache_bytes<R>(a.N, 1 << g.lpp_shift) : 0) + g.pair_bytes;
   const dim3 grid((unsigned)(g.tiles * g.nseg)), block(64);
+  // (float64: the four-wave form for the gradients of a mean, and for the others where the
+  // texel cache is on, i.e. with wide pixels)
+  constexpr bool kDouble = sizeof(S) == 8;
+  const bool w4 = kDouble && g.cache;
+#define CHOP_STRIP_BWD(CORR_)                                                               \
+  do {                                                                                      \
+    if (a.reduce == 0)                                                                      \
+      strip_backward_kernel<S, CORR_, 0, kDouble><<<grid, block, smem, stream>>>(a, g);     \
+    else if (w4)                                                                            \
+      strip_backward_kernel<S, CORR_, 1, kDouble><<<grid, block, smem, stream>>>(a, g);     \
+    else                                                                                    \
+      strip_backward_kernel<S, CORR_, 1, false><<<grid, block, smem, stream>>>(a, g);       \
+  } while (0)
   if (a.corr == BEST_GROUP_PAIR) {
-    if constexpr (sizeof(S) != 2) {
-      if (a.reduce == 0)
-        strip_backward_kernel<S, 3, 0><<<grid, block, smem, stream>>>(a, g);
-      else
-        strip_backward_kernel<S, 3, 1><<<grid, block, smem, stream>>>(a, g);
-    }
+    if constexpr (sizeof(S) != 2) CHOP_STRIP_BWD(3);
   } else if (a.corr == WARP_ONLY) {
-    strip_backward_kernel<S, 4, 0><<<grid, block, smem, stream>>>(a, g);
+    strip_backward_kernel<S, 4, 0, kDouble><<<grid, block, smem, stream>>>(a, g);
   } else if (a.corr == SUM_SQUARED_DIFFERENCE) {
-    if (a.reduce == 0)
-      strip_backward_kernel<S, 2, 0><<<grid, block, smem, stream>>>(a, g);
-    else
-      strip_backward_kernel<S, 2, 1><<<grid, block, smem, stream>>>(a, g);
+    CHOP_STRIP_BWD(2);
   } else if (a.corr == SQUARED_DIFFERENCE) {
-    if (a.reduce == 0)
-      strip_backward_kernel<S, 0, 0><<<grid, block, smem, stream>>>(a, g);
-    else
-      strip_backward_kernel<S, 0, 1><<<grid, block, smem, stream>>>(a, g);
+    CHOP_STRIP_BWD(0);
   } else {
-    if (a.reduce == 0)
-      strip_backward_kernel<S, 1, 0><<<grid, block, smem, stream>>>(a, g);
-    else
-      strip_backward_kernel<S, 1, 1><<<grid, block, smem, stream>>>(a, g);
+    CHOP_STRIP_BWD(1);
   }
+#undef CHOP_STRIP_BWD
   if ((err = hipGetLastError()) != hipSuccess) return err;
   if constexpr (sizeof(S) == 2) {
     if ((err = launch_narrow2<S>(a.ref_grad_acc, a.ref_grad, n_ref, a.src_grad_acc, a.src_grad, n_src,
