@@ -24,11 +24,12 @@
 // are merged in registers and leave as one atomic add per tap and channel when the cell
 // changes (the reference issues one per voxel) -- a run that is still open at the end of a
 // chunk waits in LDS for the view's turn in the next chunk; the per-voxel depth gradient is
-// summed over the pixel's lanes in registers and stored once.  Wide pixels (16 lanes or more:
-// at most four pixels per wave, whose atomics would each carry one pixel's channels) put a
-// small write-back cache of texels in LDS between the runs and memory: consecutive runs of a
-// pixel and its neighbours hit the same texels, and a texel leaves as one atomic per channel
-// when another texel needs its slot.
+// summed over the pixel's lanes in registers and stored once.  Wide pixels in double (16 lanes
+// or more: at most four pixels per wave, whose atomics would each carry one pixel's channels)
+// put a small write-back cache of texels in LDS between the runs and memory: consecutive runs
+// of a pixel and its neighbours hit the same texels, and a texel leaves as one atomic per
+// channel when another texel needs its slot; with the cache a run ends with its chunk (it is
+// not carried), which leaves LDS for a fourth wave per SIMD.
 #include <type_traits>
 
 #include "internal.h"
