@@ -758,6 +758,75 @@ def test_strip_many_views(oracle, C, N, dtype, reduce):
             assert_backward_close(host(g), w)
 
 
+@pytest.mark.parametrize("C,N", [(12, 3), (32, 2), (20, 1)])
+def test_strip_float64_wide_pixels(oracle, C, N):
+    """Float64 with 16 lanes or more per pixel and few views: the strip gradient kernels then put
+    a texel cache in LDS between the runs and memory, end every run with its chunk instead of
+    carrying it, and run in their four-waves-per-SIMD form.  Every op that reaches them, both
+    reduces; D = 21 leaves a ragged last chunk."""
+    B, H, W, D = 1, 11, 15, 21
+    t = reference_test_case(3, B, N, H, W, C, D, np.float64, seed=3 * C + N)
+    t["Ts"] = (t["Ts"] + np.linspace(-1, 1, N)[None, :, None]).astype(np.float64)
+    args = tuple(t[k] for k in ("ref", "src", "base_plane", "offsets", "Rs", "Ts"))
+    ins = [dev(x) for x in args]
+    rng = np.random.default_rng(C + N)
+    groups = 4
+    depth_grid = t["base_plane"] + t["offsets"][:, None, None, :]
+    a2 = (t["ref"], t["src"], depth_grid, t["Rs"], t["Ts"])
+    in2 = [dev(x) for x in a2]
+    for reduce in ("MEAN", "MIN"):
+        want_cost, want_mask = oracle.cost_volume_fwd(*args, reduce)
+        cost, mask = chop.cost_volume_raw(*ins, reduce)
+        _assert_family(2)
+        assert np.array_equal(host(mask), want_mask) and np.array_equal(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape)
+        want = oracle.cost_volume_bwd(*args, cg, want_mask, reduce)
+        got = chop.cost_volume_grad(*ins, dev(cg), mask, reduce)
+        _assert_family(2)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+
+        want_cost, want_mask = oracle.cost_volume_v2_fwd(*a2, reduce, groups)
+        cost, mask = chop.cost_volume_v2_raw(*in2, reduce, groups)
+        assert np.array_equal(host(mask), want_mask) and np.array_equal(host(cost), want_cost)
+        cg = rng.standard_normal(want_cost.shape)
+        want = oracle.cost_volume_v2_bwd(*a2, cg, want_mask, reduce, groups)
+        got = chop.cost_volume_grad_v2(*in2, dev(cg), mask, reduce, groups)
+        _assert_family(2)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+
+        want_cost, want_mask = oracle.cost_aggregate_fwd(*args, reduce)
+        cost, mask = chop.cost_aggregate_raw(*ins, reduce)
+        assert np.array_equal(host(mask), want_mask)
+        cg = rng.standard_normal(want_cost.shape)
+        want = oracle.cost_aggregate_bwd(*args, cg, want_mask, reduce)
+        got = chop.cost_aggregate_grad(*ins, dev(cg), mask, reduce)
+        _assert_family(2)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+
+        want_cost, want_mask = oracle.cost_volume_v3_fwd(*args, reduce, groups)
+        cost, mask = chop.cost_volume_v3_raw(*ins, reduce, groups)
+        assert np.array_equal(host(mask), want_mask)
+        cg = rng.standard_normal(want_cost.shape)
+        want = oracle.cost_volume_v3_bwd(*args, cg, want_mask, reduce, groups)
+        got = chop.cost_volume_grad_v3(*ins, dev(cg), mask, reduce, groups)
+        for g, w in zip(got, want):
+            assert_backward_close(host(g), w)
+
+    fargs = args[1:]
+    want_feat, want_mask = oracle.feature_aggregate_fwd(*fargs)
+    feat, mask = chop.feature_aggregate_raw(*ins[1:])
+    assert np.array_equal(host(mask), want_mask) and np.array_equal(host(feat), want_feat)
+    cg = rng.standard_normal(want_feat.shape)
+    want = oracle.feature_aggregate_bwd(*fargs, cg, want_mask)
+    got = chop.feature_aggregate_grad(*ins[1:], dev(cg), mask)
+    _assert_family(2)
+    for g, w in zip(got, want):
+        assert_backward_close(host(g), w)
+
+
 # ---- samples that jump far between consecutive depths ------------------------------------------
 @pytest.mark.parametrize("C", [4, 8, 16, 32, 64])
 def test_backward_cells_outside_the_scatter_window(oracle, C):
